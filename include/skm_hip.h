@@ -1,0 +1,158 @@
+/* C ABI of libskm_hip.so: the MI355X (gfx950) device side of the Super K-Means
+ * assign/update hot path.
+ *
+ * The reference library is header-only C++ whose per-point work is done by
+ * BLAS sgemm_, OpenMP loops and AVX/NEON kernels.  Each entry point below
+ * replaces one of those CPU routines with hand-written HIP kernels; the cited
+ * file:line is the reference routine it stands in for (paths relative to the
+ * reference's include/superkmeans/).  Host C++ (include/superkmeans/*.h) and
+ * the language bindings call only this header; no HIP type crosses it.
+ *
+ * Conventions
+ *   - every function returns 0 on success and a negative code on failure;
+ *     skm_last_error() returns the message of the calling thread's last failure;
+ *   - pointers named d_* are device pointers obtained from skm_malloc (or any
+ *     other HIP allocation on the context's device); h_* are host pointers;
+ *   - matrices are row-major fp32, indices are uint32_t, counts are uint32_t
+ *     unless stated;
+ *   - work is enqueued on the context's stream; functions that return a value
+ *     through a host pointer synchronise that stream before returning, all
+ *     others are asynchronous with respect to the host;
+ *   - a context is not thread-safe (the reference objects are not either,
+ *     superkmeans.h:132-133).
+ */
+#ifndef SKM_HIP_H
+#define SKM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SKM_OK 0
+#define SKM_ERR_INVALID (-1) /* bad argument (null pointer, zero size, size over a limit) */
+#define SKM_ERR_HIP (-2)     /* a HIP runtime call failed                                  */
+#define SKM_ERR_NO_DEVICE (-3)
+#define SKM_ERR_OOM (-4)
+
+/* Tuning constants of the reference (common.h:89-115) that shape device work. */
+#define SKM_H_DIM_SIZE 64
+#define SKM_Y_BATCH_SIZE 1024
+#define SKM_X_BATCH_SIZE 4096
+
+typedef struct skm_ctx skm_ctx;
+
+const char* skm_last_error(void);
+int skm_device_count(int* out_count);
+
+/* One context = one device + one HIP stream + reusable workspace. */
+int skm_ctx_create(int device, skm_ctx** out_ctx);
+int skm_ctx_destroy(skm_ctx* ctx);
+int skm_sync(skm_ctx* ctx);
+/* Upper bound, in bytes, of the scratch a single stage call may allocate (default 4 GiB). */
+int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
+
+/* Device memory and transfers (stand in for the reference's std::unique_ptr<float[]> buffers,
+ * superkmeans.h:191-201). */
+int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr);
+int skm_free(skm_ctx* ctx, void* d_ptr);
+int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
+int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);
+int skm_copy(skm_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
+int skm_fill_u32(skm_ctx* ctx, void* d_dst, uint32_t value, size_t count);
+
+/* Per-stage device timers, named like the reference's profiler scopes (profiler.h:296-312;
+ * "search/1st_blas", "search/blas", "search/pdx", "rotator", "update_centroids", ...).
+ * While enabled every stage brackets its kernels with events on the context's stream. */
+int skm_prof_enable(skm_ctx* ctx, int enabled);
+int skm_prof_reset(skm_ctx* ctx);
+/* Sum of device milliseconds and number of recorded intervals of one scope (synchronises). */
+int skm_prof_get(skm_ctx* ctx, const char* scope, double* out_ms, uint64_t* out_calls);
+/* Writes "name=ms/calls;" pairs for every scope seen; returns needed length incl. NUL. */
+int skm_prof_dump(skm_ctx* ctx, char* h_buf, size_t buf_len, size_t* out_needed);
+
+/* Row-wise squared L2 norms over the first `cols` columns of an rows x d matrix.
+ * cols == d : GetL2NormsRowMajor (superkmeans.h:1162-1171)
+ * cols <  d : GetPartialL2NormsRowMajor (superkmeans.h:1147-1157) */
+int skm_norms(skm_ctx* ctx, const float* d_m, size_t rows, size_t d, size_t cols, float* d_out);
+
+/* out(n x d) = X(n x d) . Q^T with Q row-major d x d: ADSamplingPruner::Rotate,
+ * pdx/adsampling.h:156-216 (sgemm_('T','N') with the pruner's matrix). MFMA GEMM. */
+int skm_rotate(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const float* d_q, float* d_out);
+/* out(n x d) = R(n x d) . Q, given Q^T (row-major transpose of Q): ADSamplingPruner::Unrotate,
+ * pdx/adsampling.h:223-299. */
+int skm_unrotate(skm_ctx* ctx, const float* d_r, size_t n, size_t d, const float* d_qt, float* d_out);
+/* out(cols x rows) = in(rows x cols)^T (used once to keep Q^T next to Q). */
+int skm_transpose(skm_ctx* ctx, const float* d_in, size_t rows, size_t cols, float* d_out);
+
+/* PDXLayout::PDXify<false> (pdx/layout.h:155-232) plus CentroidsToAuxiliaryHorizontal
+ * (superkmeans.h:1206-1212): per chunk of 1024 centroids the first vertical_d dimensions are
+ * written dimension-major, the remaining ones as 64-wide row-major blocks; d_aux (k x vertical_d)
+ * receives a dense copy of the first vertical_d columns (may be NULL).
+ * vertical_d must equal GetDimensionSplit(d).vertical_d (pdx/layout.h:115-140). */
+int skm_pdxify(skm_ctx* ctx, const float* d_c, size_t k, size_t d, size_t vertical_d, float* d_pdx,
+               float* d_aux);
+
+/* BatchComputer::FindNearestNeighbor (distance_computers/batch_computers.h:104-171): exact top-1 of
+ * every row of X among the k rows of C using ||x||^2 + ||c||^2 - 2 x.c, evaluated per batch of 1024
+ * centroids in ascending order with the reference's update rule (strict <, clamp at 0, lowest
+ * index on ties).  d_xnorm / d_cnorm are full squared norms. */
+int skm_assign_full(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, size_t k, size_t d,
+                    const float* d_xnorm, const float* d_cnorm, uint32_t* d_out_idx, float* d_out_dist);
+
+/* BatchComputer::FindNearestNeighborWithPruning (batch_computers.h:297-409) with
+ * PDXearch::Top1PartialSearchWithThresholdAndPartialDistances / Prune / SetBestCandidate
+ * (pdx/pdxearch.h:118-238,266-327).
+ *   d_c        row-major centroids (GEMM operand and seed distance, batch_computers.h:372-377)
+ *   d_pdx      the same centroids in PDX layout, d_aux their first vertical_d columns
+ *   d_ratios   d + 1 floats, ADSamplingPruner::ratios (pdx/adsampling.h:93-99)
+ *   d_xnorm_p / d_cnorm_p  squared norms over the first partial_d columns
+ *   d_inout_idx in: previous assignment (seed); out: new assignment
+ *   d_out_dist  out: squared distance to the new assignment (unclamped, as the reference)
+ *   h_out_not_pruned  sum over points of the per-point not-pruned counts (input of TunePartialD,
+ *                     superkmeans.h:1230-1241); synchronises.
+ *   h_out_stage_pairs optional array of (d - vertical_d) / 64 + 2 counters: live (point, centroid)
+ *                     pairs entering each pruning step (algorithmic-bytes accounting); may be NULL. */
+int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, const float* d_pdx,
+                      const float* d_aux, size_t k, size_t d, size_t vertical_d, uint32_t partial_d,
+                      const float* d_ratios, const float* d_xnorm_p, const float* d_cnorm_p,
+                      uint32_t* d_inout_idx, float* d_out_dist, uint64_t* h_out_not_pruned,
+                      uint64_t* h_out_stage_pairs);
+
+/* SuperKMeans::UpdateCentroids (superkmeans.h:729-765): sums[c] = sum of rows assigned to c, taken
+ * in ascending point order per centroid exactly like the reference's per-thread scan, and
+ * sizes[c] = number of such rows.  No floating-point atomics: point ids are stably sorted by
+ * assignment and each centroid's segment is reduced by one workgroup. */
+int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_t* d_idx, size_t k,
+               float* d_out_sums, uint32_t* d_out_sizes);
+/* First loop of SuperKMeans::ConsolidateCentroids (superkmeans.h:940-951): c *= float(1.0 / size)
+ * for every non-empty cluster. */
+int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d);
+/* SuperKMeans::PostprocessCentroids (superkmeans.h:1357-1371): c /= ||c||. */
+int skm_normalize_rows(skm_ctx* ctx, float* d_c, size_t k, size_t d);
+/* Row edits of SplitClusters (superkmeans.h:905-920; hierarchical_superkmeans.h:606-625,665-673),
+ * applied in list order.  op[4*i] = kind (0: copy row src->dst then perturb dst by (1 +/- eps) and
+ * src by (1 -/+ eps) alternating per column; 1: dst = (w * dst + src) / (w + 1)), op[4*i+1] = dst,
+ * op[4*i+2] = src, op[4*i+3] = bit pattern of float w. */
+int skm_edit_rows(skm_ctx* ctx, float* d_c, size_t d, const uint32_t* h_ops, size_t n_ops);
+/* SuperKMeans::ComputeCost (superkmeans.h:973-981): sum of n distances, accumulated in fp64 with a
+ * fixed reduction tree. */
+int skm_wcss(skm_ctx* ctx, const float* d_dist, size_t n, double* h_out_cost);
+/* SuperKMeans::ComputeShift (superkmeans.h:988-998): sum_c ||new_c - prev_c||^2. */
+int skm_shift(skm_ctx* ctx, const float* d_new, const float* d_prev, size_t k, size_t d,
+              double* h_out_shift);
+/* HierarchicalSuperKMeans::CompactMesoclusterToBuffer (hierarchical_superkmeans.h:685-704):
+ * out[j] = X[index[j]], norms_out[j] = norms_in[index[j]] (norm pointers may be NULL). */
+int skm_gather_rows(skm_ctx* ctx, const float* d_x, size_t d, const uint64_t* d_index, size_t m,
+                    float* d_out, const float* d_norms_in, float* d_norms_out);
+/* GetTrueAssignmentsFromIndirectionBuffer (hierarchical_superkmeans.h:763-779):
+ * out[index[j]] = local[j] + offset. */
+int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_t* d_local, size_t m,
+                            uint32_t offset, uint32_t* d_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SKM_HIP_H */

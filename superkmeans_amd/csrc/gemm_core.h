@@ -1,0 +1,192 @@
+// fp32 MFMA GEMM core for gfx950 (CDNA4): D[m][n] = sum_k A[m][k] * B[n][k].
+//
+// Both operands are row-major with the reduction dimension contiguous, which is
+// exactly the shape of every dense product on the Super K-Means hot path:
+//   * distances  x . c     (reference: batch_computers.h:47-83, sgemm_('T','N'))
+//   * rotation   X . Q^T   (reference: pdx/adsampling.h:191-215)
+// One workgroup (256 threads = 4 wavefronts of 64) owns a 128 x 128 tile of D,
+// each wavefront a 64 x 64 quadrant held as 2 x 2 accumulators of the
+// v_mfma_f32_32x32x2_f32 instruction.  Operand slices of BK = 32 columns are
+// staged through LDS (double buffered, row stride 36 floats so that both the
+// 16-byte stores and the 16-byte fragment reads are bank-conflict free).
+//
+// The k index inside a group of 8 columns is permuted so that one ds_read_b128
+// per operand fragment feeds four consecutive MFMAs: lane l supplies columns
+// (l / 32) * 4 + i to the i-th MFMA for both A and B, which is a valid GEMM
+// because A and B use the same permutation.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace skm {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int GEMM_TM = 128;
+constexpr int GEMM_TN = 128;
+constexpr int GEMM_BK = 32;
+constexpr int GEMM_LDS_STRIDE = GEMM_BK + 4;
+constexpr int GEMM_THREADS = 256;
+constexpr int GEMM_XCDS = 8;
+
+struct GemmOperands {
+    const float* A;  // M x K, row stride lda
+    const float* B;  // N x K, row stride ldb
+    int M, N, K;
+    int64_t lda, ldb;
+    int tiles_m, tiles_n;
+};
+
+// Accumulators of one wavefront: acc[mb][nb] is a 32 x 32 block.  Element r of
+// acc[mb][nb] held by lane l is D[m][n] with
+//   m = wave_m0 + mb * 32 + 8 * (r / 4) + 4 * (l / 32) + (r % 4)
+//   n = wave_n0 + nb * 32 + (l % 32)
+struct WaveAcc {
+    floatx16 v[2][2];
+};
+
+__device__ __forceinline__ int acc_row(int mb, int r, int lane) {
+    return mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+}
+__device__ __forceinline__ int acc_col(int nb, int lane) {
+    return nb * 32 + (lane & 31);
+}
+
+// Maps the hardware workgroup id to a tile so that the workgroups resident on
+// one XCD (ids congruent mod 8 are dispatched to the same XCD) cover a compact
+// block of 8 M-tiles x several N-tiles and share operand panels in that XCD's L2.
+__device__ __forceinline__ void tile_of_block(const GemmOperands& g, int bid, int& tm, int& tn) {
+    const int total = g.tiles_m * g.tiles_n;
+    const int q = total / GEMM_XCDS, r = total % GEMM_XCDS;
+    const int x = bid % GEMM_XCDS, within = bid / GEMM_XCDS;
+    const int L = x * q + (x < r ? x : r) + within;
+    const int band_tiles = 8 * g.tiles_n;
+    const int band = L / band_tiles;
+    const int in_band = L - band * band_tiles;
+    const int rows_in_band = (g.tiles_m - band * 8) < 8 ? (g.tiles_m - band * 8) : 8;
+    tn = in_band / rows_in_band;
+    tm = band * 8 + in_band % rows_in_band;
+}
+
+template <bool VEC>
+__device__ __forceinline__ floatx4 load_k4(const float* row, int k, int K) {
+    floatx4 v;
+    if (VEC) {
+        if (k + 3 < K) {
+            v = *reinterpret_cast<const floatx4*>(row + k);
+        } else {
+            v.x = (k + 0 < K) ? row[k + 0] : 0.0f;
+            v.y = (k + 1 < K) ? row[k + 1] : 0.0f;
+            v.z = (k + 2 < K) ? row[k + 2] : 0.0f;
+            v.w = 0.0f;
+        }
+    } else {
+        v.x = (k + 0 < K) ? row[k + 0] : 0.0f;
+        v.y = (k + 1 < K) ? row[k + 1] : 0.0f;
+        v.z = (k + 2 < K) ? row[k + 2] : 0.0f;
+        v.w = (k + 3 < K) ? row[k + 3] : 0.0f;
+    }
+    return v;
+}
+
+// Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are
+// 16-byte aligned so operand slices can be fetched with dwordx4 loads.
+template <bool VEC>
+__device__ __forceinline__ void gemm_tile(
+    const GemmOperands& g, int tm, int tn, float* lds, WaveAcc& acc
+) {
+    float* As = lds;                                    // [2][TM * STRIDE]
+    float* Bs = lds + 2 * GEMM_TM * GEMM_LDS_STRIDE;    // [2][TN * STRIDE]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // Global -> register staging: thread covers rows (tid / 8) + 32 * p, 4 floats at column 4 * (tid % 8).
+    const int ld_row = tid >> 3;
+    const int ld_k = (tid & 7) * 4;
+    const float* a_rows[4];
+    const float* b_rows[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        int ra = tm * GEMM_TM + ld_row + 32 * p;
+        int rb = tn * GEMM_TN + ld_row + 32 * p;
+        ra = ra < g.M ? ra : g.M - 1;  // clamp: duplicates are masked by the epilogue
+        rb = rb < g.N ? rb : g.N - 1;
+        a_rows[p] = g.A + (int64_t) ra * g.lda;
+        b_rows[p] = g.B + (int64_t) rb * g.ldb;
+    }
+    floatx4 ra[4], rb[4];
+
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
+
+    const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;
+
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        ra[p] = load_k4<VEC>(a_rows[p], ld_k, g.K);
+        rb[p] = load_k4<VEC>(b_rows[p], ld_k, g.K);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        *reinterpret_cast<floatx4*>(&As[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = ra[p];
+        *reinterpret_cast<floatx4*>(&Bs[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = rb[p];
+    }
+    __syncthreads();
+
+    const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        const bool more = (kt + 1) < nk;
+        if (more) {
+            const int k0 = (kt + 1) * GEMM_BK + ld_k;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                ra[p] = load_k4<VEC>(a_rows[p], k0, g.K);
+                rb[p] = load_k4<VEC>(b_rows[p], k0, g.K);
+            }
+        }
+        const float* as = As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off;
+        const float* bs = Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off;
+#pragma unroll
+        for (int kg = 0; kg < GEMM_BK / 8; ++kg) {
+            floatx4 a0 = *reinterpret_cast<const floatx4*>(as + kg * 8);
+            floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + kg * 8);
+            floatx4 b0 = *reinterpret_cast<const floatx4*>(bs + kg * 8);
+            floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + kg * 8);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
+                acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
+                acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
+                acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
+            }
+        }
+        if (more) {
+            float* asn = As + (cur ^ 1) * GEMM_TM * GEMM_LDS_STRIDE;
+            float* bsn = Bs + (cur ^ 1) * GEMM_TN * GEMM_LDS_STRIDE;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                *reinterpret_cast<floatx4*>(&asn[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = ra[p];
+                *reinterpret_cast<floatx4*>(&bsn[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = rb[p];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+constexpr int GEMM_LDS_FLOATS = 2 * (GEMM_TM + GEMM_TN) * GEMM_LDS_STRIDE;
+
+inline bool gemm_operands_vectorizable(const GemmOperands& g) {
+    return (reinterpret_cast<uintptr_t>(g.A) % 16 == 0) && (reinterpret_cast<uintptr_t>(g.B) % 16 == 0) &&
+           (g.lda % 4 == 0) && (g.ldb % 4 == 0);
+}
+
+} // namespace skm

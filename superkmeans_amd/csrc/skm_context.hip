@@ -1,0 +1,284 @@
+// Context, memory, error and profiler plumbing of libskm_hip.so.
+#include "skm_internal.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+namespace skm {
+
+static thread_local char g_last_error[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return SKM_OK;
+    const int code = (e == hipErrorOutOfMemory) ? SKM_ERR_OOM : SKM_ERR_HIP;
+    return set_error(code, "HIP error %d (%s) in %s", (int) e, hipGetErrorString(e), what);
+}
+
+int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out) {
+    if (slot < 0 || slot >= 4) return set_error(SKM_ERR_INVALID, "bad workspace slot");
+    if (ctx->ws_bytes[slot] < bytes) {
+        if (ctx->ws[slot]) {
+            SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            SKM_HIP_TRY(hipFree(ctx->ws[slot]));
+            ctx->ws[slot] = nullptr;
+            ctx->ws_bytes[slot] = 0;
+        }
+        size_t want = bytes + bytes / 8;
+        hipError_t e = hipMalloc(&ctx->ws[slot], want);
+        if (e != hipSuccess) {
+            want = bytes;
+            SKM_HIP_TRY(hipMalloc(&ctx->ws[slot], want));
+        }
+        ctx->ws_bytes[slot] = want;
+    }
+    *out = ctx->ws[slot];
+    return SKM_OK;
+}
+
+int pinned(skm_ctx* ctx, size_t bytes, void** out) {
+    if (ctx->h_pinned_bytes < bytes) {
+        if (ctx->h_pinned) {
+            SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            SKM_HIP_TRY(hipHostFree(ctx->h_pinned));
+            ctx->h_pinned = nullptr;
+            ctx->h_pinned_bytes = 0;
+        }
+        SKM_HIP_TRY(hipHostMalloc(&ctx->h_pinned, bytes, hipHostMallocDefault));
+        ctx->h_pinned_bytes = bytes;
+    }
+    *out = ctx->h_pinned;
+    return SKM_OK;
+}
+
+static hipEvent_t take_event(skm_ctx* ctx) {
+    if (!ctx->event_pool.empty()) {
+        hipEvent_t e = ctx->event_pool.back();
+        ctx->event_pool.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) return nullptr;
+    return e;
+}
+
+ScopedStage::ScopedStage(skm_ctx* ctx, const char* scope) : ctx_(ctx) {
+    if (!ctx->prof) return;
+    iv_.scope = scope;
+    iv_.start = take_event(ctx);
+    iv_.stop = take_event(ctx);
+    if (!iv_.start || !iv_.stop) return;
+    if (hipEventRecord(iv_.start, ctx->stream) != hipSuccess) return;
+    active_ = true;
+}
+
+ScopedStage::~ScopedStage() {
+    if (!active_) return;
+    if (hipEventRecord(iv_.stop, ctx_->stream) != hipSuccess) return;
+    ctx_->pending.push_back(iv_);
+    if (ctx_->pending.size() >= 4096) resolve_pending(ctx_);
+}
+
+int resolve_pending(skm_ctx* ctx) {
+    if (ctx->pending.empty()) return SKM_OK;
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    for (auto& iv : ctx->pending) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, iv.start, iv.stop) == hipSuccess) {
+            auto& t = ctx->timers[iv.scope];
+            t.ms += ms;
+            t.calls += 1;
+        }
+        ctx->event_pool.push_back(iv.start);
+        ctx->event_pool.push_back(iv.stop);
+    }
+    ctx->pending.clear();
+    return SKM_OK;
+}
+
+__global__ void fill_u32_kernel(uint32_t* dst, uint32_t value, size_t count) {
+    size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t) gridDim.x * blockDim.x;
+    for (; i < count; i += stride) dst[i] = value;
+}
+
+} // namespace skm
+
+using namespace skm;
+
+extern "C" {
+
+const char* skm_last_error(void) { return g_last_error; }
+
+int skm_device_count(int* out_count) {
+    if (!out_count) return set_error(SKM_ERR_INVALID, "skm_device_count: null output");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *out_count = 0;
+        return set_error(SKM_ERR_NO_DEVICE, "no HIP device: %s", hipGetErrorString(e));
+    }
+    *out_count = n;
+    return SKM_OK;
+}
+
+int skm_ctx_create(int device, skm_ctx** out_ctx) {
+    if (!out_ctx) return set_error(SKM_ERR_INVALID, "skm_ctx_create: null output");
+    *out_ctx = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0)
+        return set_error(SKM_ERR_NO_DEVICE, "skm_ctx_create: no HIP device is visible");
+    if (device < 0 || device >= n)
+        return set_error(SKM_ERR_INVALID, "skm_ctx_create: device %d out of range [0,%d)", device, n);
+    SKM_HIP_TRY(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    SKM_HIP_TRY(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(SKM_ERR_NO_DEVICE, "skm_ctx_create: device %d is %s; this library is built for gfx950 only",
+                         device, prop.gcnArchName);
+    skm_ctx* ctx = new skm_ctx();
+    ctx->device = device;
+    hipError_t e = hipStreamCreate(&ctx->stream);
+    if (e != hipSuccess) {
+        delete ctx;
+        return check_hip(e, "hipStreamCreate");
+    }
+    *out_ctx = ctx;
+    return SKM_OK;
+}
+
+int skm_ctx_destroy(skm_ctx* ctx) {
+    if (!ctx) return SKM_OK;
+    hipSetDevice(ctx->device);
+    hipStreamSynchronize(ctx->stream);
+    for (auto& iv : ctx->pending) {
+        hipEventDestroy(iv.start);
+        hipEventDestroy(iv.stop);
+    }
+    for (auto e : ctx->event_pool) hipEventDestroy(e);
+    for (int i = 0; i < 4; ++i)
+        if (ctx->ws[i]) hipFree(ctx->ws[i]);
+    if (ctx->h_pinned) hipHostFree(ctx->h_pinned);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return SKM_OK;
+}
+
+int skm_sync(skm_ctx* ctx) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SKM_OK;
+}
+
+int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(bytes >= (size_t(64) << 20), "workspace limit must be at least 64 MiB");
+    ctx->workspace_limit = bytes;
+    return SKM_OK;
+}
+
+int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr) {
+    SKM_REQUIRE(ctx && out_d_ptr, "null argument");
+    *out_d_ptr = nullptr;
+    if (bytes == 0) bytes = 16;
+    SKM_HIP_TRY(hipSetDevice(ctx->device));
+    SKM_HIP_TRY(hipMalloc(out_d_ptr, bytes));
+    return SKM_OK;
+}
+
+int skm_free(skm_ctx* ctx, void* d_ptr) {
+    SKM_REQUIRE(ctx, "null context");
+    if (!d_ptr) return SKM_OK;
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    SKM_HIP_TRY(hipFree(d_ptr));
+    return SKM_OK;
+}
+
+int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    if (bytes == 0) return SKM_OK;
+    SKM_REQUIRE(d_dst && h_src, "null pointer");
+    SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SKM_OK;
+}
+
+int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    if (bytes == 0) return SKM_OK;
+    SKM_REQUIRE(h_dst && d_src, "null pointer");
+    SKM_HIP_TRY(hipMemcpyAsync(h_dst, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SKM_OK;
+}
+
+int skm_copy(skm_ctx* ctx, void* d_dst, const void* d_src, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    if (bytes == 0) return SKM_OK;
+    SKM_REQUIRE(d_dst && d_src, "null pointer");
+    SKM_HIP_TRY(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return SKM_OK;
+}
+
+int skm_fill_u32(skm_ctx* ctx, void* d_dst, uint32_t value, size_t count) {
+    SKM_REQUIRE(ctx, "null context");
+    if (count == 0) return SKM_OK;
+    SKM_REQUIRE(d_dst, "null pointer");
+    size_t blocks = (count + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned) blocks), dim3(256), 0, ctx->stream,
+                       (uint32_t*) d_dst, value, count);
+    return check_hip(hipGetLastError(), "fill_u32_kernel launch");
+}
+
+int skm_prof_enable(skm_ctx* ctx, int enabled) {
+    SKM_REQUIRE(ctx, "null context");
+    if (!enabled) SKM_TRY(resolve_pending(ctx));
+    ctx->prof = enabled != 0;
+    return SKM_OK;
+}
+
+int skm_prof_reset(skm_ctx* ctx) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_TRY(resolve_pending(ctx));
+    ctx->timers.clear();
+    return SKM_OK;
+}
+
+int skm_prof_get(skm_ctx* ctx, const char* scope, double* out_ms, uint64_t* out_calls) {
+    SKM_REQUIRE(ctx && scope, "null argument");
+    SKM_TRY(resolve_pending(ctx));
+    auto it = ctx->timers.find(scope);
+    if (out_ms) *out_ms = (it == ctx->timers.end()) ? 0.0 : it->second.ms;
+    if (out_calls) *out_calls = (it == ctx->timers.end()) ? 0 : it->second.calls;
+    return SKM_OK;
+}
+
+int skm_prof_dump(skm_ctx* ctx, char* h_buf, size_t buf_len, size_t* out_needed) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_TRY(resolve_pending(ctx));
+    std::string s;
+    char tmp[256];
+    for (auto& kv : ctx->timers) {
+        snprintf(tmp, sizeof(tmp), "%s=%.6f/%llu;", kv.first.c_str(), kv.second.ms,
+                 (unsigned long long) kv.second.calls);
+        s += tmp;
+    }
+    if (out_needed) *out_needed = s.size() + 1;
+    if (h_buf && buf_len > 0) {
+        size_t ncopy = s.size() < buf_len - 1 ? s.size() : buf_len - 1;
+        memcpy(h_buf, s.data(), ncopy);
+        h_buf[ncopy] = '\0';
+    }
+    return SKM_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,101 @@
+// Internal glue shared by the translation units of libskm_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "skm_hip.h"
+
+struct skm_scope_timer {
+    double ms = 0.0;
+    uint64_t calls = 0;
+};
+
+struct skm_pending_interval {
+    std::string scope;
+    hipEvent_t start, stop;
+};
+
+struct skm_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    size_t workspace_limit = size_t(4) << 30;
+    // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
+    void* ws[4] = {nullptr, nullptr, nullptr, nullptr};
+    size_t ws_bytes[4] = {0, 0, 0, 0};
+    // Small pinned host buffer for scalar results.
+    void* h_pinned = nullptr;
+    size_t h_pinned_bytes = 0;
+    bool prof = false;
+    std::map<std::string, skm_scope_timer> timers;
+    std::vector<skm_pending_interval> pending;
+    std::vector<hipEvent_t> event_pool;
+};
+
+namespace skm {
+
+int set_error(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+
+#define SKM_HIP_TRY(expr)                                                                          \
+    do {                                                                                           \
+        int _rc = ::skm::check_hip((expr), #expr);                                                 \
+        if (_rc != SKM_OK) return _rc;                                                             \
+    } while (0)
+
+#define SKM_TRY(expr)                                                                              \
+    do {                                                                                           \
+        int _rc = (expr);                                                                          \
+        if (_rc != SKM_OK) return _rc;                                                             \
+    } while (0)
+
+#define SKM_REQUIRE(cond, msg)                                                                     \
+    do {                                                                                           \
+        if (!(cond)) return ::skm::set_error(SKM_ERR_INVALID, "%s: %s", __func__, msg);           \
+    } while (0)
+
+// Returns a scratch buffer of at least `bytes` for slot `slot` (grow-only).
+int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out);
+int pinned(skm_ctx* ctx, size_t bytes, void** out);
+
+// RAII device timer for one profiler scope; no-op unless profiling is enabled.
+class ScopedStage {
+  public:
+    ScopedStage(skm_ctx* ctx, const char* scope);
+    ~ScopedStage();
+
+  private:
+    skm_ctx* ctx_;
+    bool active_ = false;
+    skm_pending_interval iv_;
+};
+
+int resolve_pending(skm_ctx* ctx);
+
+// ---- launchers implemented in the kernel translation units ----
+
+// D = A . B^T stored row-major (ldo), optionally turned into squared distances
+// out[m][n] = -2 * D[m][n] + row_norm[m] + col_norm[n] when both norm pointers are non-null.
+int launch_gemm_store(skm_ctx* ctx, const float* A, int M, int64_t lda, const float* B, int N,
+                      int64_t ldb, int K, float* out, int64_t ldo, const float* row_norm,
+                      const float* col_norm);
+
+// Per (granule of 64 centroids, point) minimum of -2 x.c + |x|^2 + |c|^2 and its lowest index,
+// written as uint2 {float bits, index} to granule_min[granule * n + point].
+int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int n, int d,
+                       int64_t ldc, int64_t ldx, const float* xnorm, const float* cnorm,
+                       uint2* granule_min);
+
+int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, uint32_t* out_idx,
+                          float* out_dist);
+
+int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
+                 const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
+                 int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
+                 unsigned long long* d_counters);
+
+} // namespace skm
