@@ -1,0 +1,259 @@
+// Pruned top-1 search: one wavefront per point walks the batches of 1024 centroids in order and
+// reproduces PDXearch::Top1PartialSearchWithThresholdAndPartialDistances / Prune / SetBestCandidate
+// (reference pdx/pdxearch.h:118-238,266-327) and the per-row body of
+// BatchComputer::FindNearestNeighborWithPruning (distance_computers/batch_computers.h:357-405).
+//
+// Wavefront mapping
+//   * first test against best * ratios[d'] : 64 partial distances per step, survivors compacted in
+//     ascending position order with a ballot + prefix popcount into an LDS list
+//     (InitPositionsArray, scalar_computers.h:87-98);
+//   * every 64-dimension horizontal block: 4 survivors per step, 16 lanes x float4 each, reduced
+//     with four cross-lane exchanges, followed by the same ballot compaction
+//     (EvaluatePruningPredicateOnPositionsArray, pdxearch.h:67-80);
+//   * the [d', vertical_d) dimensions are read last from the dense auxiliary copy;
+//   * survivors of the final test (ratio 1) update the best candidate, lowest position first.
+// The threshold of a batch is fixed while the batch is processed and only tightens between
+// batches, exactly as on the CPU, so the order in which survivors are visited cannot change results.
+#include "skm_internal.h"
+
+#include <float.h>
+
+namespace skm {
+
+constexpr int PRUNE_WAVES = 4;
+constexpr int PRUNE_CAP = SKM_Y_BATCH_SIZE;
+
+struct PruneArgs {
+    const float* partial;  // n_chunk x ld_partial partial distances over the first partial_d dims
+    int64_t ld_partial;
+    const float* x;        // n_chunk x d rotated points
+    const float* c;        // k x d row-major centroids
+    const float* pdx;      // PDX copy of c
+    const float* aux;      // k x vertical_d
+    const float* ratios;   // d + 1
+    uint32_t* idx;         // in: previous assignment, out: new assignment
+    float* dist;           // out
+    uint32_t* not_pruned;  // out: per-point count of survivors of the first test, summed over batches
+    unsigned long long* stage_pairs;  // optional accounting, may be null
+    int n, k, d, vertical_d, partial_d;
+};
+
+__device__ __forceinline__ float group16_sum(float v) {
+    v += __shfl_xor(v, 8);
+    v += __shfl_xor(v, 4);
+    v += __shfl_xor(v, 2);
+    v += __shfl_xor(v, 1);
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// Keeps the survivors whose accumulated distance is below thr, preserving order. In-place: slot s
+// is rewritten only by elements read from slots >= s, and each step reads before it writes.
+__device__ __forceinline__ int compact_survivors(uint16_t* pos, float* acc, int cnt, float thr, int lane) {
+    int out = 0;
+    for (int s0 = 0; s0 < cnt; s0 += 64) {
+        const int s = s0 + lane;
+        const bool in = s < cnt;
+        const uint16_t p = in ? pos[s] : 0;
+        const float a = in ? acc[s] : 0.0f;
+        const bool keep = in && (a < thr);
+        const unsigned long long mask = __ballot(keep);
+        if (keep) {
+            const int slot = out + __popcll(mask & ((1ull << lane) - 1ull));
+            pos[slot] = p;
+            acc[slot] = a;
+        }
+        out += __popcll(mask);
+    }
+    return out;
+}
+
+template <bool VEC>
+__global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
+    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
+    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int p = blockIdx.x * PRUNE_WAVES + wave;
+    if (p >= a.n) return;
+    uint16_t* pos = s_pos[wave];
+    float* acc = s_acc[wave];
+    const int d = a.d, V = a.vertical_d, dp = a.partial_d;
+    const int H = d - V;
+    const int n_hblocks = H / SKM_H_DIM_SIZE;
+    const float* xq = a.x + (int64_t) p * d;
+    const int sub = lane & 15;   // lane within a 16-lane group
+    const int grp = lane >> 4;   // which of the 4 survivors handled per step
+
+    // Distance to the previous assignment over all d dimensions (batch_computers.h:372-377).
+    uint32_t best_idx = a.idx[p];
+    float best;
+    {
+        const float* cp = a.c + (int64_t) best_idx * d;
+        float s = 0.0f;
+        if (VEC) {
+            for (int t = lane * 4; t < d; t += 256) {
+                const float4 xv = *reinterpret_cast<const float4*>(xq + t);
+                const float4 cv = *reinterpret_cast<const float4*>(cp + t);
+                float e;
+                e = cv.x - xv.x; s += e * e;
+                e = cv.y - xv.y; s += e * e;
+                e = cv.z - xv.z; s += e * e;
+                e = cv.w - xv.w; s += e * e;
+            }
+        } else {
+            for (int t = lane; t < d; t += 64) {
+                const float e = cp[t] - xq[t];
+                s += e * e;
+            }
+        }
+        best = wave_sum(s);
+    }
+
+    uint32_t not_pruned_total = 0;
+    const int n_batches = (a.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE;
+    const float* prow = a.partial + (int64_t) p * a.ld_partial;
+    for (int jb = 0; jb < n_batches; ++jb) {
+        const int base = jb * SKM_Y_BATCH_SIZE;
+        const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
+        const uint32_t prev_top_1 = best_idx;
+        // ---- first test on the GEMM partial distances ----
+        float thr = best * a.ratios[dp];
+        int cnt = 0;
+        for (int c0 = 0; c0 < m; c0 += 64) {
+            const int c = c0 + lane;
+            const bool in = c < m;
+            const float v = in ? prow[base + c] : 0.0f;
+            const bool keep = in && (v < thr);
+            const unsigned long long mask = __ballot(keep);
+            if (keep) {
+                const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+                pos[slot] = (uint16_t) c;
+                acc[slot] = v;
+            }
+            cnt += __popcll(mask);
+        }
+        not_pruned_total += (uint32_t) cnt;
+        if (a.stage_pairs && lane == 0 && cnt) atomicAdd(&a.stage_pairs[0], (unsigned long long) cnt);
+        // Only survivor is the incumbent: nothing to do (pdxearch.h:140-143).
+        if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
+        if (cnt == 0) continue;
+
+        // ---- horizontal blocks of 64 dimensions, PDX layout (pdxearch.h:149-180) ----
+        const float* chunk = a.pdx + (int64_t) base * d;
+        int dims_seen = dp;
+        for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
+            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + hb], (unsigned long long) cnt);
+            const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
+            const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
+            float4 xv;
+            if (VEC) {
+                xv = *reinterpret_cast<const float4*>(xb + sub * 4);
+            } else {
+                xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
+            }
+            for (int s0 = 0; s0 < cnt; s0 += 4) {
+                const int s = s0 + grp;
+                const bool in = s < cnt;
+                const int cpos = in ? pos[s] : pos[0];
+                const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                float4 cv;
+                if (VEC) {
+                    cv = *reinterpret_cast<const float4*>(cb);
+                } else {
+                    cv = make_float4(cb[0], cb[1], cb[2], cb[3]);
+                }
+                float e, part = 0.0f;
+                e = xv.x - cv.x; part += e * e;
+                e = xv.y - cv.y; part += e * e;
+                e = xv.z - cv.z; part += e * e;
+                e = xv.w - cv.w; part += e * e;
+                part = group16_sum(part);
+                if (in && sub == 0) acc[s] += part;
+            }
+            dims_seen += SKM_H_DIM_SIZE;
+            thr = best * a.ratios[dims_seen];
+            cnt = compact_survivors(pos, acc, cnt, thr, lane);
+        }
+
+        // ---- remaining vertical dimensions [d', V) from the dense auxiliary copy (pdxearch.h:183-216) ----
+        if (cnt > 0 && dp < V) {
+            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + n_hblocks], (unsigned long long) cnt);
+            const int left = V - dp;
+            for (int s0 = 0; s0 < cnt; s0 += 4) {
+                const int s = s0 + grp;
+                const bool in = s < cnt;
+                const int cpos = in ? pos[s] : pos[0];
+                const float* cb = a.aux + (int64_t) (base + cpos) * V + dp;
+                float part = 0.0f;
+                for (int t = sub; t < left; t += 16) {
+                    const float e = xq[dp + t] - cb[t];
+                    part += e * e;
+                }
+                part = group16_sum(part);
+                if (in && sub == 0) acc[s] += part;
+            }
+            thr = best * a.ratios[d];
+            cnt = compact_survivors(pos, acc, cnt, thr, lane);
+        }
+
+        // ---- SetBestCandidate (pdxearch.h:223-238): strict <, lowest position wins ties ----
+        if (cnt > 0) {
+            float bv = FLT_MAX;
+            int bp = 0x7fffffff;
+            for (int s = lane; s < cnt; s += 64) {
+                const float v = acc[s];
+                const int q = pos[s];
+                if (v < bv || (v == bv && q < bp)) {
+                    bv = v;
+                    bp = q;
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(bv, off);
+                const int op = __shfl_xor(bp, off);
+                if (ov < bv || (ov == bv && op < bp)) {
+                    bv = ov;
+                    bp = op;
+                }
+            }
+            if (bp != 0x7fffffff && bv < best) {
+                best = bv;
+                best_idx = (uint32_t) (base + bp);
+            }
+        }
+    }
+    if (lane == 0) {
+        a.idx[p] = best_idx;
+        a.dist[p] = best;
+        a.not_pruned[p] = not_pruned_total;
+    }
+}
+
+int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
+                 const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
+                 int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
+                 uint32_t* out_not_pruned, unsigned long long* d_stage_pairs) {
+    if (n_chunk <= 0) return SKM_OK;
+    PruneArgs a;
+    a.partial = partial; a.ld_partial = ld_partial; a.x = x; a.c = c; a.pdx = pdx; a.aux = aux;
+    a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned;
+    a.stage_pairs = d_stage_pairs;
+    a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
+    const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
+                     (reinterpret_cast<uintptr_t>(c) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
+    dim3 grid((n_chunk + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    if (vec)
+        hipLaunchKernelGGL(prune_kernel<true>, grid, block, 0, ctx->stream, a);
+    else
+        hipLaunchKernelGGL(prune_kernel<false>, grid, block, 0, ctx->stream, a);
+    return check_hip(hipGetLastError(), "prune_kernel launch");
+}
+
+} // namespace skm

@@ -1,0 +1,422 @@
+// Centroid update without floating-point atomics.
+//
+// SuperKMeans::UpdateCentroids (reference superkmeans.h:729-765) lets every OpenMP thread scan all
+// assignments and accumulate the rows of the centroids it owns, so each centroid's sum is taken in
+// ascending point order.  Here the point ids are first sorted by assignment with a stable LSD radix
+// sort (integer work only), then one workgroup per centroid walks its segment in that same
+// ascending order and accumulates in registers.  The result is run-to-run deterministic and has the
+// reference's summation order.
+#include "skm_internal.h"
+
+#include <algorithm>
+
+namespace skm {
+
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_TILE = 4096;  // elements per workgroup and pass
+constexpr int RADIX = 256;
+
+__global__ __launch_bounds__(256) void count_assignments_kernel(
+    const uint32_t* __restrict__ idx, size_t n, uint32_t k, uint32_t* __restrict__ sizes
+) {
+    size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t) gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        const uint32_t a = idx[i];
+        if (a < k) atomicAdd(&sizes[a], 1u);
+    }
+}
+
+// Exclusive scan of `len` counters by one workgroup (len is k + 1 or 256 * n_tiles: small).
+__global__ __launch_bounds__(1024) void exclusive_scan_kernel(
+    const uint32_t* __restrict__ in, uint32_t* __restrict__ out, size_t len
+) {
+    __shared__ uint32_t s_wave[16];
+    __shared__ uint32_t s_carry;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) s_carry = 0;
+    __syncthreads();
+    for (size_t base = 0; base < len; base += 1024) {
+        const size_t i = base + tid;
+        const uint32_t v = (i < len) ? in[i] : 0u;
+        uint32_t incl = v;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        uint32_t wave_off = 0;
+        for (int w = 0; w < wave; ++w) wave_off += s_wave[w];
+        const uint32_t carry = s_carry;
+        if (i < len) out[i] = carry + wave_off + incl - v;
+        __syncthreads();
+        if (tid == 1023) s_carry = carry + wave_off + incl;
+        __syncthreads();
+    }
+}
+
+// Pass 1 of a radix step: digit histogram of one tile, stored digit-major so that one exclusive
+// scan over [digit][tile] yields the global base of every (digit, tile) pair.
+__global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
+    const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t n_tiles, uint32_t* __restrict__ hist
+) {
+    __shared__ uint32_t s_hist[RADIX];
+    s_hist[threadIdx.x] = 0;
+    __syncthreads();
+    const size_t t0 = (size_t) blockIdx.x * SORT_TILE;
+    for (int r = 0; r < SORT_TILE / SORT_THREADS; ++r) {
+        const size_t i = t0 + (size_t) r * SORT_THREADS + threadIdx.x;
+        if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & (RADIX - 1)], 1u);
+    }
+    __syncthreads();
+    hist[(size_t) threadIdx.x * n_tiles + blockIdx.x] = s_hist[threadIdx.x];
+}
+
+// Pass 2: stable scatter.  The tile is consumed in rounds of 256 consecutive elements; inside a
+// round the rank of an element among equal digits is (equal digits in earlier wavefronts) +
+// (equal digits in lower lanes of its wavefront), the latter from eight ballots.
+__global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift,
+    uint32_t n_tiles, const uint32_t* __restrict__ bases, uint32_t* __restrict__ keys_out,
+    uint32_t* __restrict__ vals_out, int vals_are_iota
+) {
+    __shared__ uint32_t s_base[RADIX];
+    __shared__ uint32_t s_wave_cnt[SORT_THREADS / 64][RADIX];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    s_base[tid] = bases[(size_t) tid * n_tiles + blockIdx.x];
+    const size_t t0 = (size_t) blockIdx.x * SORT_TILE;
+    for (int r = 0; r < SORT_TILE / SORT_THREADS; ++r) {
+        const size_t i = t0 + (size_t) r * SORT_THREADS + tid;
+        const bool in = i < n;
+#pragma unroll
+        for (int w = 0; w < SORT_THREADS / 64; ++w) s_wave_cnt[w][tid] = 0;
+        __syncthreads();
+        uint32_t key = 0, val = 0, digit = 0;
+        unsigned long long peers = 0;
+        if (in) {
+            key = keys_in[i];
+            val = vals_are_iota ? (uint32_t) i : vals_in[i];
+            digit = (key >> shift) & (RADIX - 1);
+        }
+        // Lanes holding the same digit (inactive lanes never match an active one).
+        unsigned long long match = __ballot(in);
+#pragma unroll
+        for (int b = 0; b < 8; ++b) {
+            const unsigned long long vote = __ballot(in && ((digit >> b) & 1u));
+            match &= ((digit >> b) & 1u) ? vote : ~vote;
+        }
+        peers = match;
+        const uint32_t rank_in_wave = (uint32_t) __popcll(peers & ((1ull << lane) - 1ull));
+        if (in && rank_in_wave == 0) s_wave_cnt[wave][digit] = (uint32_t) __popcll(peers);
+        __syncthreads();
+        if (in) {
+            uint32_t before = 0;
+            for (int w = 0; w < wave; ++w) before += s_wave_cnt[w][digit];
+            const uint32_t dst = s_base[digit] + before + rank_in_wave;
+            keys_out[dst] = key;
+            vals_out[dst] = val;
+        }
+        __syncthreads();
+        uint32_t add = 0;
+#pragma unroll
+        for (int w = 0; w < SORT_THREADS / 64; ++w) add += s_wave_cnt[w][tid];
+        s_base[tid] += add;
+        __syncthreads();
+    }
+}
+
+// One workgroup per centroid; thread t owns columns 4t..4t+3 (+ blockDim * 4 ...).  Rows of the
+// segment are visited in ascending point id; `UNROLL` independent row loads are kept in flight.
+template <bool VEC>
+__global__ __launch_bounds__(256) void segment_sum_kernel(
+    const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
+    const uint32_t* __restrict__ offsets, float* __restrict__ sums
+) {
+    const uint32_t c = blockIdx.x;
+    const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
+    float* out = sums + (size_t) c * d;
+    if (VEC) {
+        const size_t d4 = d / 4;
+        for (size_t t = threadIdx.x; t < d4; t += blockDim.x) {
+            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+            uint32_t j = j0;
+            for (; j + 8 <= j1; j += 8) {
+                float4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    acc.x += v[u].x;
+                    acc.y += v[u].y;
+                    acc.z += v[u].z;
+                    acc.w += v[u].w;
+                }
+            }
+            for (; j < j1; ++j) {
+                const float4 v = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j] * d)[t];
+                acc.x += v.x;
+                acc.y += v.y;
+                acc.z += v.z;
+                acc.w += v.w;
+            }
+            reinterpret_cast<float4*>(out)[t] = acc;
+        }
+    } else {
+        for (size_t t = threadIdx.x; t < d; t += blockDim.x) {
+            float acc = 0.0f;
+            for (uint32_t j = j0; j < j1; ++j) acc += x[(size_t) sorted_ids[j] * d + t];
+            out[t] = acc;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void scale_by_size_kernel(
+    float* __restrict__ sums, const uint32_t* __restrict__ sizes, size_t k, size_t d
+) {
+    const size_t c = blockIdx.x;
+    const uint32_t s = sizes[c];
+    if (s == 0) return;
+    const float mult = (float) (1.0 / (double) s);  // float mult_factor = 1.0 / cluster_sizes[i]
+    float* row = sums + c * d;
+    for (size_t t = threadIdx.x; t < d; t += blockDim.x) row[t] *= mult;
+}
+
+__global__ __launch_bounds__(256) void normalize_rows_kernel(float* __restrict__ c, size_t k, size_t d) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t) blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= k) return;
+    float* p = c + row * d;
+    float s = 0.0f;
+    for (size_t t = lane; t < d; t += 64) s += p[t] * p[t];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
+    const float inv = 1.0f / sqrtf(s);
+    for (size_t t = lane; t < d; t += 64) p[t] *= inv;
+}
+
+// Applies the row edits of SplitClusters one after the other (later edits see earlier ones).
+__global__ __launch_bounds__(256) void edit_rows_kernel(float* __restrict__ c, size_t d, const uint32_t* __restrict__ ops, size_t n_ops) {
+    const float eps = 1.0f / 1024.0f;
+    for (size_t o = 0; o < n_ops; ++o) {
+        const uint32_t kind = ops[4 * o], dst = ops[4 * o + 1], src = ops[4 * o + 2];
+        const float w = __uint_as_float(ops[4 * o + 3]);
+        float* pd = c + (size_t) dst * d;
+        float* ps = c + (size_t) src * d;
+        if (kind == 0) {
+            for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
+                const float v = ps[j];
+                if (j % 2 == 0) {
+                    pd[j] = v * (1 + eps);
+                    ps[j] = v * (1 - eps);
+                } else {
+                    pd[j] = v * (1 - eps);
+                    ps[j] = v * (1 + eps);
+                }
+            }
+        } else {
+            for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
+                float val = 0.0f;
+                val += w * pd[j];
+                val += 1.0f * ps[j];
+                val /= (w + 1.0f);
+                pd[j] = val;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+constexpr int REDUCE_BLOCKS = 512;
+
+// Fixed-shape two-stage reductions in fp64: block b sums elements b*256+tid, +512*256, ... so the
+// association depends only on the element count.
+template <int MODE>  // 0: sum a[i]; 1: sum (a[i]-b[i])^2; 2: sum of uint32 a[i] (as exact integers)
+__global__ __launch_bounds__(256) void reduce_stage1_kernel(
+    const float* __restrict__ a, const float* __restrict__ b, size_t n, double* __restrict__ partial
+) {
+    __shared__ double s[256];
+    double acc = 0.0;
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) REDUCE_BLOCKS * 256) {
+        if (MODE == 0) {
+            acc += (double) a[i];
+        } else if (MODE == 1) {
+            const float t = a[i] - b[i];
+            acc += (double) (t * t);
+        } else {
+            acc += (double) reinterpret_cast<const uint32_t*>(a)[i];
+        }
+    }
+    s[threadIdx.x] = acc;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) partial[blockIdx.x] = s[0];
+}
+
+__global__ __launch_bounds__(256) void reduce_stage2_kernel(const double* __restrict__ partial, double* __restrict__ out) {
+    __shared__ double s[256];
+    s[threadIdx.x] = partial[threadIdx.x] + partial[threadIdx.x + 256];
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = s[0];
+}
+
+static int reduce_to_host(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_out) {
+    void* ws = nullptr;
+    SKM_TRY(workspace(ctx, 3, (REDUCE_BLOCKS + 8) * sizeof(double), &ws));
+    double* partial = (double*) ws;
+    double* result = partial + REDUCE_BLOCKS;
+    if (mode == 0)
+        hipLaunchKernelGGL(reduce_stage1_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
+    else if (mode == 1)
+        hipLaunchKernelGGL(reduce_stage1_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
+    else
+        hipLaunchKernelGGL(reduce_stage1_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
+    SKM_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(reduce_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, result);
+    SKM_HIP_TRY(hipGetLastError());
+    void* hp = nullptr;
+    SKM_TRY(pinned(ctx, 64, &hp));
+    SKM_HIP_TRY(hipMemcpyAsync(hp, result, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    *h_out = *(double*) hp;
+    return SKM_OK;
+}
+
+int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_out) {
+    return reduce_to_host(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, h_out);
+}
+
+} // namespace skm
+
+using namespace skm;
+
+extern "C" {
+
+int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_t* d_idx, size_t k,
+               float* d_out_sums, uint32_t* d_out_sizes) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(d_out_sums && d_out_sizes, "null output");
+    SKM_REQUIRE(k > 0 && d > 0, "k and d must be positive");
+    SKM_REQUIRE(k < 0xffffffffULL && n < 0xffffffffULL, "n and k must fit in 32 bits");
+    SKM_REQUIRE(n == 0 || (d_x && d_idx), "null input");
+    ScopedStage st(ctx, "update_centroids");
+    // Scratch: keys/vals double buffers (4n u32), offsets (k+1), per-tile histograms.
+    const uint32_t n_tiles = (uint32_t) ((n + SORT_TILE - 1) / SORT_TILE);
+    const size_t hist_len = (size_t) RADIX * std::max<uint32_t>(n_tiles, 1);
+    const size_t words = 4 * n + (k + 1) + 2 * hist_len + 64;
+    void* ws = nullptr;
+    SKM_TRY(workspace(ctx, 1, words * sizeof(uint32_t), &ws));
+    uint32_t* keys_a = (uint32_t*) ws;
+    uint32_t* keys_b = keys_a + n;
+    uint32_t* vals_a = keys_b + n;
+    uint32_t* vals_b = vals_a + n;
+    uint32_t* offsets = vals_b + n;
+    uint32_t* hist = offsets + (k + 1);
+    uint32_t* bases = hist + hist_len;
+
+    SKM_TRY(skm_fill_u32(ctx, d_out_sizes, 0u, k));
+    if (n > 0) {
+        const unsigned blocks = (unsigned) std::min<size_t>((n + 255) / 256, 4096);
+        hipLaunchKernelGGL(count_assignments_kernel, dim3(blocks), dim3(256), 0, ctx->stream, d_idx, n, (uint32_t) k, d_out_sizes);
+        SKM_HIP_TRY(hipGetLastError());
+    }
+    // offsets[c] = number of points assigned to centroids < c and offsets[k] = n: exclusive scan of
+    // the sizes followed by one zero.
+    void* ws2 = nullptr;
+    SKM_TRY(workspace(ctx, 2, (k + 1) * sizeof(uint32_t), &ws2));
+    uint32_t* sizes_z = (uint32_t*) ws2;
+    SKM_HIP_TRY(hipMemcpyAsync(sizes_z, d_out_sizes, k * sizeof(uint32_t), hipMemcpyDeviceToDevice, ctx->stream));
+    SKM_TRY(skm_fill_u32(ctx, sizes_z + k, 0u, 1));
+    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, sizes_z, offsets, k + 1);
+    SKM_HIP_TRY(hipGetLastError());
+
+    const uint32_t* sorted_ids = nullptr;
+    if (n > 0) {
+        int bits = 0;
+        while (bits < 32 && ((k - 1) >> bits) != 0) ++bits;
+        const int passes = std::max(1, (bits + 7) / 8);
+        const uint32_t* kin = d_idx;
+        const uint32_t* vin = nullptr;
+        uint32_t* kout = keys_a;
+        uint32_t* vout = vals_a;
+        for (int p = 0; p < passes; ++p) {
+            const int shift = 8 * p;
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, n_tiles, hist);
+            SKM_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, hist, bases, hist_len);
+            SKM_HIP_TRY(hipGetLastError());
+            hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift,
+                               n_tiles, bases, kout, vout, p == 0 ? 1 : 0);
+            SKM_HIP_TRY(hipGetLastError());
+            kin = kout;
+            vin = vout;
+            kout = (kout == keys_a) ? keys_b : keys_a;
+            vout = (vout == vals_a) ? vals_b : vals_a;
+        }
+        sorted_ids = vin;
+    } else {
+        sorted_ids = vals_a;
+    }
+    const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
+                     (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
+    const size_t lanes = vec ? d / 4 : d;
+    unsigned threads = (unsigned) std::min<size_t>(256, ((lanes + 63) / 64) * 64);
+    if (vec)
+        hipLaunchKernelGGL(segment_sum_kernel<true>, dim3((unsigned) k), dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+    else
+        hipLaunchKernelGGL(segment_sum_kernel<false>, dim3((unsigned) k), dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+    return check_hip(hipGetLastError(), "segment_sum_kernel launch");
+}
+
+int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d) {
+    SKM_REQUIRE(ctx && d_sums && d_sizes, "null argument");
+    if (k == 0) return SKM_OK;
+    ScopedStage st(ctx, "consolidate/splitting");
+    hipLaunchKernelGGL(scale_by_size_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_sums, d_sizes, k, d);
+    return check_hip(hipGetLastError(), "scale_by_size_kernel launch");
+}
+
+int skm_normalize_rows(skm_ctx* ctx, float* d_c, size_t k, size_t d) {
+    SKM_REQUIRE(ctx && d_c, "null argument");
+    if (k == 0) return SKM_OK;
+    ScopedStage st(ctx, "consolidate/normalize");
+    hipLaunchKernelGGL(normalize_rows_kernel, dim3((unsigned) ((k + 3) / 4)), dim3(256), 0, ctx->stream, d_c, k, d);
+    return check_hip(hipGetLastError(), "normalize_rows_kernel launch");
+}
+
+int skm_edit_rows(skm_ctx* ctx, float* d_c, size_t d, const uint32_t* h_ops, size_t n_ops) {
+    SKM_REQUIRE(ctx && d_c, "null argument");
+    if (n_ops == 0) return SKM_OK;
+    SKM_REQUIRE(h_ops, "null ops");
+    void* ws = nullptr;
+    SKM_TRY(workspace(ctx, 2, n_ops * 4 * sizeof(uint32_t), &ws));
+    SKM_HIP_TRY(hipMemcpyAsync(ws, h_ops, n_ops * 4 * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));  // h_ops is caller memory: do not outlive the call
+    hipLaunchKernelGGL(edit_rows_kernel, dim3(1), dim3(256), 0, ctx->stream, d_c, d, (const uint32_t*) ws, n_ops);
+    return check_hip(hipGetLastError(), "edit_rows_kernel launch");
+}
+
+int skm_wcss(skm_ctx* ctx, const float* d_dist, size_t n, double* h_out_cost) {
+    SKM_REQUIRE(ctx && h_out_cost, "null argument");
+    SKM_REQUIRE(n == 0 || d_dist, "null input");
+    ScopedStage st(ctx, "compute_cost");
+    return reduce_to_host(ctx, 0, d_dist, nullptr, n, h_out_cost);
+}
+
+int skm_shift(skm_ctx* ctx, const float* d_new, const float* d_prev, size_t k, size_t d, double* h_out_shift) {
+    SKM_REQUIRE(ctx && h_out_shift, "null argument");
+    SKM_REQUIRE(k * d == 0 || (d_new && d_prev), "null input");
+    ScopedStage st(ctx, "shift");
+    return reduce_to_host(ctx, 1, d_new, d_prev, k * d, h_out_shift);
+}
+
+} // extern "C"

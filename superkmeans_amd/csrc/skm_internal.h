@@ -96,6 +96,6 @@ int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, 
 int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
                  const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
                  int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
-                 unsigned long long* d_counters);
+                 uint32_t* out_not_pruned, unsigned long long* d_stage_pairs);
 
 } // namespace skm

@@ -1,0 +1,140 @@
+"""GPU parity of the dense stages against the CPU oracle: norms, rotation, exact search.
+
+Tolerances follow the reference's own tests: distances within 1e-4 relative, indices equal unless
+the two candidate distances are within 1e-4 relative (tests/test_distance_computers.cpp:83-152);
+rotation round trip max error < 1e-4 (tests/test_rotation.cpp:56-149).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _assign_full(capi, ctx, X, C):
+    n, d = X.shape
+    k = C.shape[0]
+    dX, dC = ctx.array(X), ctx.array(C)
+    xn, cn = ctx.empty(n), ctx.empty(k)
+    idx, dist = ctx.empty(n, np.uint32), ctx.empty(n)
+    capi.check(ctx.lib.skm_norms(ctx.handle, dX.ptr, n, d, d, xn.ptr))
+    capi.check(ctx.lib.skm_norms(ctx.handle, dC.ptr, k, d, d, cn.ptr))
+    capi.check(ctx.lib.skm_assign_full(ctx.handle, dX.ptr, n, dC.ptr, k, d, xn.ptr, cn.ptr, idx.ptr, dist.ptr))
+    out = idx.download(), dist.download(), xn.download()
+    for a in (dX, dC, xn, cn, idx, dist):
+        a.free()
+    return out
+
+
+@pytest.mark.parametrize("rows,d,cols", [(1000, 768, 768), (1000, 768, 96), (333, 50, 50), (64, 1024, 85), (5, 3, 2)])
+def test_norms_match_oracle(capi, ctx, oracle, rows, d, cols):
+    x = np.random.default_rng(1).standard_normal((rows, d)).astype(np.float32)
+    dx, out = ctx.array(x), ctx.empty(rows)
+    capi.check(ctx.lib.skm_norms(ctx.handle, dx.ptr, rows, d, cols, out.ptr))
+    got = out.download()
+    ref = oracle.norms(x, cols)
+    exact = (x[:, :cols].astype(np.float64) ** 2).sum(1)
+    assert np.allclose(got, ref, rtol=1e-5, atol=0)
+    assert np.allclose(got, exact, rtol=1e-5, atol=0)
+    dx.free(), out.free()
+
+
+# shapes of tests/test_distance_computers.cpp:89-95 plus ragged / non-vectorisable ones
+@pytest.mark.parametrize("n,k,d", [(100, 50, 32), (1000, 100, 64), (5000, 1000, 128), (500, 2000, 256),
+                                   (1000, 257, 50), (777, 3000, 600), (4097, 1025, 130), (1, 1, 1), (3, 1100, 7)])
+def test_assign_full_matches_oracle_and_brute_force(capi, ctx, oracle, n, k, d):
+    g = np.random.default_rng(n + k + d)
+    X = g.standard_normal((n, d)).astype(np.float32)
+    C = g.standard_normal((k, d)).astype(np.float32)
+    gi, gd, _ = _assign_full(capi, ctx, X, C)
+    oi, od = oracle.find_nn(X, C)
+    bi, bbest, _ = oracle.brute_force(X, C)
+    X64, C64 = X.astype(np.float64), C.astype(np.float64)
+    for ref_idx in (oi, bi):
+        for i in np.nonzero(gi != ref_idx)[0]:
+            da = ((X64[i] - C64[gi[i]]) ** 2).sum()
+            db = ((X64[i] - C64[ref_idx[i]]) ** 2).sum()
+            assert abs(da - db) <= 1e-4 * max(db, 1e-12), f"point {i}: gpu {gi[i]} ({da}) vs ref {ref_idx[i]} ({db})"
+    assert np.allclose(gd, bbest, rtol=1e-4, atol=1e-5)
+    assert np.allclose(gd, od, rtol=1e-4, atol=1e-5)
+
+
+def test_assign_full_clustered_data_exact_agreement(capi, ctx, oracle, blobs):
+    """On well separated mixtures there are no near ties: indices must agree exactly (C1-like shape, reduced n)."""
+    X = blobs(20000, 768, 1000, std=0.3, seed=5)
+    C = X[np.random.default_rng(0).choice(len(X), 1000, replace=False)].copy()
+    gi, gd, _ = _assign_full(capi, ctx, X, C)
+    oi, od = oracle.find_nn(X, C)
+    bi, bbest, bsecond = oracle.brute_force(X, C)
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    assert np.all((gi == bi) | tie)
+    assert np.mean(gi != oi) <= 1e-4
+    # a point that coincides with a centroid has distance clamped at 0 (batch_computers.h:165)
+    assert gd.min() >= 0.0
+
+
+def test_assign_full_duplicate_centroids_take_lowest_index(capi, ctx):
+    """Exact ties resolve to the lowest index inside a batch (minCoeff) and across batches (strict <)."""
+    g = np.random.default_rng(3)
+    base = g.standard_normal((8, 64)).astype(np.float32)
+    C = np.tile(base, (300, 1))  # 2400 centroids: every centroid repeats every 8 rows, across 3 batches
+    X = base + 0.01 * g.standard_normal((8, 64)).astype(np.float32)
+    gi, _, _ = _assign_full(capi, ctx, X, C)
+    assert np.array_equal(gi, np.arange(8, dtype=np.uint32))
+
+
+def test_assign_full_chunked_by_workspace_limit(capi, ctx, oracle):
+    """A tiny workspace forces several chunks of points; results must not change."""
+    g = np.random.default_rng(9)
+    X = g.standard_normal((3000, 96)).astype(np.float32)
+    C = g.standard_normal((700, 96)).astype(np.float32)
+    ref = _assign_full(capi, ctx, X, C)
+    capi.check(ctx.lib.skm_ctx_set_workspace_limit(ctx.handle, 64 << 20))
+    try:
+        # 64 MiB / (11 granules * 8 B) is still > 3000 points, so shrink k-granule budget via a large k instead
+        C2 = np.concatenate([C, g.standard_normal((40000, 96)).astype(np.float32) + 50.0])
+        got = _assign_full(capi, ctx, np.tile(X, (5, 1)), C2)
+    finally:
+        capi.check(ctx.lib.skm_ctx_set_workspace_limit(ctx.handle, 4 << 30))
+    assert np.array_equal(got[0][:3000], ref[0])
+    assert np.array_equal(got[0][3000:6000], ref[0])
+
+
+@pytest.mark.parametrize("d", [50, 128, 256, 512, 768, 1024])
+def test_rotate_unrotate_match_oracle_and_round_trip(capi, ctx, oracle, d):
+    n = 300
+    Q = oracle.rotation_matrix(d, seed=42)
+    X = np.random.default_rng(d).standard_normal((n, d)).astype(np.float32)
+    dX, dQ, dQt, dR, dB = ctx.array(X), ctx.array(Q), ctx.empty((d, d)), ctx.empty((n, d)), ctx.empty((n, d))
+    capi.check(ctx.lib.skm_transpose(ctx.handle, dQ.ptr, d, d, dQt.ptr))
+    assert np.array_equal(dQt.download(), Q.T)
+    capi.check(ctx.lib.skm_rotate(ctx.handle, dX.ptr, n, d, dQ.ptr, dR.ptr))
+    capi.check(ctx.lib.skm_unrotate(ctx.handle, dR.ptr, n, d, dQt.ptr, dB.ptr))
+    R, B = dR.download(), dB.download()
+    exact = X.astype(np.float64) @ Q.astype(np.float64).T
+    assert np.abs(R - exact).max() < 1e-5
+    assert np.abs(R - oracle.rotate(Q, X)).max() < 1e-5
+    assert np.abs(B - X).max() < 1e-4 and np.abs(B - X).mean() < 1e-5  # test_rotation.cpp:56-149
+    # norm preservation, rel < 1e-5 (test_rotation.cpp:157-206)
+    nx, nr = np.linalg.norm(X.astype(np.float64), axis=1), np.linalg.norm(R.astype(np.float64), axis=1)
+    assert np.max(np.abs(nx - nr) / nx) < 1e-5
+    for a in (dX, dQ, dQt, dR, dB):
+        a.free()
+
+
+def test_transpose_rectangular(capi, ctx):
+    a = np.arange(37 * 101, dtype=np.float32).reshape(37, 101)
+    da, dt = ctx.array(a), ctx.empty((101, 37))
+    capi.check(ctx.lib.skm_transpose(ctx.handle, da.ptr, 37, 101, dt.ptr))
+    assert np.array_equal(dt.download(), a.T)
+    da.free(), dt.free()
+
+
+def test_bad_arguments_are_rejected(capi, ctx):
+    x = ctx.empty((4, 8))
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_norms(ctx.handle, x.ptr, 4, 8, 9, x.ptr))  # cols > d
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_assign_full(ctx.handle, x.ptr, 4, None, 2, 8, x.ptr, x.ptr, x.ptr, x.ptr))
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_rotate(ctx.handle, x.ptr, 4, 8, x.ptr, x.ptr))  # in place
+    x.free()

@@ -1,0 +1,183 @@
+"""GPU parity of the HBM-bound stages against the CPU oracle: PDX relayout, gather/scatter,
+centroid update, scaling, WCSS, shift, row edits.  Integer / copy work is compared bit-exactly;
+the centroid sums are bit-exact too because the device visits each centroid's points in the same
+ascending order as the reference (superkmeans.h:742-750)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("k,d", [(1024, 128), (2048, 256), (2500, 256), (500, 768), (10000, 1024), (1, 64), (1030, 600), (300, 100)])
+def test_pdxify_bit_exact(capi, ctx, oracle, k, d):
+    C = np.random.default_rng(k + d).standard_normal((k, d)).astype(np.float32)
+    _, V = oracle.dimension_split(d)
+    dC, dP, dA = ctx.array(C), ctx.empty(k * d), ctx.empty((k, V))
+    capi.check(ctx.lib.skm_pdxify(ctx.handle, dC.ptr, k, d, V, dP.ptr, dA.ptr))
+    assert np.array_equal(dP.download(), oracle.pdxify(C))
+    assert np.array_equal(dA.download(), C[:, :V])
+    for a in (dC, dP, dA):
+        a.free()
+
+
+def test_pdxify_rejects_bad_split(capi, ctx):
+    x = ctx.empty((8, 128))
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_pdxify(ctx.handle, x.ptr, 8, 128, 60, x.ptr, None))
+    x.free()
+
+
+@pytest.mark.parametrize("n,d,k,nthreads", [(5000, 128, 100, 1), (20000, 256, 1000, 8), (3000, 50, 7, 3), (10000, 1024, 300, 8),
+                                            (70000, 64, 70000, 8), (257, 1536, 1, 2)])
+def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
+    g = np.random.default_rng(n + d)
+    X = g.standard_normal((n, d)).astype(np.float32)
+    a = g.integers(0, k, n).astype(np.uint32)
+    if k > 3:
+        a[a == 2] = 3  # force an empty cluster
+    dX, dA, dS, dZ = ctx.array(X), ctx.array(a), ctx.empty((k, d)), ctx.empty(k, np.uint32)
+    capi.check(ctx.lib.skm_update(ctx.handle, dX.ptr, n, d, dA.ptr, k, dS.ptr, dZ.ptr))
+    sums, sizes = dS.download(), dZ.download()
+    rs, rz = oracle.update_centroids(X, a, k, scale=False, n_threads=nthreads)
+    assert np.array_equal(sizes, rz)
+    assert np.array_equal(sizes, np.bincount(a, minlength=k).astype(np.uint32))
+    assert np.array_equal(sums, rs)  # same summation order as the reference -> identical bits
+    capi.check(ctx.lib.skm_scale_by_size(ctx.handle, dS.ptr, dZ.ptr, k, d))
+    means = dS.download()
+    rm, _ = oracle.update_centroids(X, a, k, scale=True, n_threads=nthreads)
+    assert np.array_equal(means, rm)
+    # closed form: fp64 mean of the assigned rows
+    for c in np.unique(a)[:20]:
+        exact = X[a == c].astype(np.float64).mean(0)
+        assert np.allclose(means[c], exact, rtol=1e-4, atol=1e-5)
+    for arr in (dX, dA, dS, dZ):
+        arr.free()
+
+
+def test_update_is_run_to_run_deterministic(capi, ctx):
+    g = np.random.default_rng(0)
+    X = g.standard_normal((50000, 96)).astype(np.float32)
+    a = g.integers(0, 64, 50000).astype(np.uint32)
+    dX, dA, dS, dZ = ctx.array(X), ctx.array(a), ctx.empty((64, 96)), ctx.empty(64, np.uint32)
+    outs = []
+    for _ in range(3):
+        capi.check(ctx.lib.skm_update(ctx.handle, dX.ptr, 50000, 96, dA.ptr, 64, dS.ptr, dZ.ptr))
+        outs.append(dS.download())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    for arr in (dX, dA, dS, dZ):
+        arr.free()
+
+
+def test_wcss_and_shift(capi, ctx):
+    import ctypes
+
+    g = np.random.default_rng(4)
+    dist = g.random(1_000_003).astype(np.float32)
+    dd = ctx.array(dist)
+    out = ctypes.c_double()
+    capi.check(ctx.lib.skm_wcss(ctx.handle, dd.ptr, dist.size, ctypes.byref(out)))
+    assert abs(out.value - dist.astype(np.float64).sum()) <= 1e-9 * dist.size
+    a = g.standard_normal((777, 130)).astype(np.float32)
+    b = g.standard_normal((777, 130)).astype(np.float32)
+    da, db = ctx.array(a), ctx.array(b)
+    capi.check(ctx.lib.skm_shift(ctx.handle, da.ptr, db.ptr, 777, 130, ctypes.byref(out)))
+    exact = ((a.astype(np.float64) - b.astype(np.float64)) ** 2).sum()
+    assert abs(out.value - exact) <= 1e-6 * exact
+    capi.check(ctx.lib.skm_wcss(ctx.handle, dd.ptr, 0, ctypes.byref(out)))
+    assert out.value == 0.0
+    for arr in (dd, da, db):
+        arr.free()
+
+
+def test_gather_rows_and_scatter_assignments(capi, ctx):
+    g = np.random.default_rng(6)
+    X = g.standard_normal((5000, 200)).astype(np.float32)
+    norms = g.random(5000).astype(np.float32)
+    index = g.permutation(5000)[:1234].astype(np.uint64)
+    dX, dN, dI = ctx.array(X), ctx.array(norms), ctx.array(index)
+    dO, dNo = ctx.empty((1234, 200)), ctx.empty(1234)
+    capi.check(ctx.lib.skm_gather_rows(ctx.handle, dX.ptr, 200, dI.ptr, 1234, dO.ptr, dN.ptr, dNo.ptr))
+    assert np.array_equal(dO.download(), X[index])
+    assert np.array_equal(dNo.download(), norms[index])
+    local = g.integers(0, 50, 1234).astype(np.uint32)
+    dL = ctx.array(local)
+    full = np.full(5000, 0xFFFFFFFF, dtype=np.uint32)
+    dF = ctx.array(full)
+    capi.check(ctx.lib.skm_scatter_assignments(ctx.handle, dI.ptr, dL.ptr, 1234, 700, dF.ptr))
+    expect = full.copy()
+    expect[index] = local + 700
+    assert np.array_equal(dF.download(), expect)
+    for arr in (dX, dN, dI, dO, dNo, dL, dF):
+        arr.free()
+
+
+def test_edit_rows_matches_split_clusters(capi, ctx, oracle):
+    """The copy+perturb edit reproduces SplitClusters' row arithmetic (superkmeans.h:905-920)."""
+    g = np.random.default_rng(8)
+    k, d = 12, 64
+    C = g.standard_normal((k, d)).astype(np.float32)
+    sizes = np.full(k, 100, dtype=np.uint32)
+    sizes[[3, 7]] = 0
+    sizes[0] = 100 + 200
+    n = int(sizes.sum())
+    rc, rs, nsplit = oracle.split_clusters(C, sizes, n, seed=42, hierarchical=False)
+    assert nsplit == 2
+    # recover which rows were split from the oracle result: dst rows are 3 and 7; find their sources
+    ops = []
+    cur = C.copy()
+    for dst in (3, 7):
+        src = None
+        for cand in range(k):
+            if cand in (3, 7) and cur[cand].tolist() == C[cand].tolist() and sizes[cand] == 0:
+                continue
+            trial = cur[cand].copy()
+            sign = np.where(np.arange(d) % 2 == 0, 1.0, -1.0).astype(np.float32)
+            if np.array_equal(trial * (np.float32(1) + sign * np.float32(1 / 1024)), rc[dst]) or True:
+                pass
+        # the oracle's choice is visible from the size bookkeeping
+        changed = [c for c in range(k) if rs[c] != sizes[c] and c not in (3, 7)]
+        src = changed[0] if len(changed) == 1 else None
+        assert src is not None or len(changed) >= 1
+        src = changed[0]
+        ops += [0, dst, src, 0]
+        break
+    # apply both edits with the same source the oracle used (sizes show a single donor twice or two donors)
+    donors = [c for c in range(k) if rs[c] != sizes[c] and c not in (3, 7)]
+    if len(donors) == 1:
+        ops = [0, 3, donors[0], 0, 0, 7, donors[0], 0]
+    else:
+        # two donors: order by which copy matches
+        ops = None
+        for d0, d1 in ((donors[0], donors[1]), (donors[1], donors[0])):
+            dC = ctx.array(C)
+            o = np.array([0, 3, d0, 0, 0, 7, d1, 0], dtype=np.uint32)
+            capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, o.ctypes.data, 2))
+            got = dC.download()
+            dC.free()
+            if np.array_equal(got, rc):
+                ops = o
+                break
+        assert ops is not None
+        return
+    dC = ctx.array(C)
+    o = np.array(ops, dtype=np.uint32)
+    capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, o.ctypes.data, len(o) // 4))
+    assert np.array_equal(dC.download(), rc)
+    dC.free()
+
+
+def test_edit_rows_balancing_and_normalize(capi, ctx):
+    g = np.random.default_rng(10)
+    C = g.standard_normal((5, 96)).astype(np.float32)
+    w = np.float32(3.0)
+    o = np.array([1, 2, 4, w.view(np.uint32)], dtype=np.uint32)
+    dC = ctx.array(C)
+    capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, 96, o.ctypes.data, 1))
+    got = dC.download()
+    exp = C.copy()
+    exp[2] = (np.float32(0) + w * C[2] + np.float32(1) * C[4]) / (w + np.float32(1))
+    assert np.array_equal(got, exp)
+    capi.check(ctx.lib.skm_normalize_rows(ctx.handle, dC.ptr, 5, 96))
+    nrm = np.linalg.norm(dC.download().astype(np.float64), axis=1)
+    assert np.allclose(nrm, 1.0, atol=1e-5)  # test_superkmeans.cpp:376-407
+    dC.free()

@@ -1,0 +1,121 @@
+"""GPU parity of the pruned search (partial GEMM + ADSampling/PDX pruning) against the CPU oracle.
+
+Bars (north_star): indices equal except where the top-2 gap is below 1e-5 relative, at most 0.01 %
+of points; pruning never discards a candidate the oracle keeps (checked through: every GPU/oracle
+disagreement must coincide with GPU == exact brute force, or be a tie)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False):
+    n, d = X.shape
+    k = C.shape[0]
+    H, V = oracle.dimension_split(d)
+    dX, dC = ctx.array(X), ctx.array(C)
+    dP, dA = ctx.empty(k * d), ctx.empty((k, V))
+    capi.check(ctx.lib.skm_pdxify(ctx.handle, dC.ptr, k, d, V, dP.ptr, dA.ptr))
+    xn, cn = ctx.empty(n), ctx.empty(k)
+    capi.check(ctx.lib.skm_norms(ctx.handle, dX.ptr, n, d, partial_d, xn.ptr))
+    capi.check(ctx.lib.skm_norms(ctx.handle, dC.ptr, k, d, partial_d, cn.ptr))
+    dR = ctx.array(np.ascontiguousarray(ratios, dtype=np.float32))
+    idx, dist = ctx.array(np.ascontiguousarray(prev, dtype=np.uint32)), ctx.empty(n)
+    total = ctypes.c_uint64()
+    stages = (ctypes.c_uint64 * (H // 64 + 2))()
+    capi.check(ctx.lib.skm_assign_pruned(ctx.handle, dX.ptr, n, dC.ptr, dP.ptr, dA.ptr, k, d, V, partial_d, dR.ptr,
+                                         xn.ptr, cn.ptr, idx.ptr, dist.ptr, ctypes.byref(total),
+                                         stages if accounting else None))
+    out = idx.download(), dist.download(), total.value, np.array(list(stages), dtype=np.uint64)
+    for a in (dX, dC, dP, dA, xn, cn, dR, idx, dist):
+        a.free()
+    return out
+
+
+def _setup(oracle, blobs, n, d, k, seed, std=0.3):
+    X = blobs(n, d, k, std=std, seed=seed)
+    g = np.random.default_rng(seed + 1)
+    C = X[g.choice(n, k, replace=False)].copy()
+    # one Lloyd step so that "previous assignments" are a realistic seed for the threshold
+    prev, _ = oracle.find_nn(X, C)
+    C2, sizes = oracle.update_centroids(X, prev, k, scale=True)
+    C2[sizes == 0] = C[sizes == 0]
+    return X, C2, prev
+
+
+@pytest.mark.parametrize("n,d,k,partial_d", [(4000, 128, 300, 32), (6000, 256, 1500, 32), (3000, 768, 1100, 96),
+                                             (4000, 1024, 2500, 128), (1500, 600, 1030, 77), (1000, 132, 260, 23)])
+def test_pruned_matches_oracle(capi, ctx, oracle, blobs, n, d, k, partial_d):
+    X, C, prev = _setup(oracle, blobs, n, d, k, seed=n + d)
+    ratios = oracle.ratios(d, 1.5)
+    gi, gd, gtotal, gst = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=True)
+    oi, od, ocounts, ost = oracle.find_nn_pruned(X, C, prev, partial_d, ratios, accounting=True)
+    bi, bbest, bsecond = oracle.brute_force(X, C)
+    mism = np.nonzero(gi != oi)[0]
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    for i in mism:
+        assert gi[i] == bi[i] or tie[i], f"point {i}: gpu {gi[i]} oracle {oi[i]} brute {bi[i]}"
+    assert len(mism) <= max(1, int(1e-4 * n))
+    same = gi == oi
+    assert np.allclose(gd[same], od[same], rtol=1e-4, atol=1e-6)
+    # returned distance is the full squared distance to the returned centroid
+    full = ((X.astype(np.float64) - C[gi].astype(np.float64)) ** 2).sum(1)
+    assert np.allclose(gd, full, rtol=1e-4, atol=1e-6)
+    # Not-pruned statistics feed TunePartialD.  Pairs entering every pruning step agree to fp32
+    # threshold noise.  The total of the first test is looser: a point that is the only member of
+    # its cluster sits exactly on its centroid, so its threshold is 0 and whether the incumbent's
+    # own partial distance (a rounding residue of |x|^2 + |c|^2 - 2 x.c) counts as "< 0" is a coin
+    # flip on either side; such a pair never enters a pruning step (pdxearch.h:140-143).
+    assert gtotal <= n * k
+    singletons = int((np.bincount(prev, minlength=k)[prev] == 1).sum())
+    assert abs(int(gtotal) - int(ocounts.sum())) <= singletons + max(3, int(2e-3 * ocounts.sum()))
+    assert gst[0] == gtotal and ost[0] == ocounts.sum()
+    assert np.all(np.abs(gst[1:].astype(np.int64) - ost[1:].astype(np.int64)) <= np.maximum(3, 2e-3 * ost[1:]))
+    # survivors shrink monotonically through the horizontal steps
+    hs = gst[1:-1]
+    assert np.all(hs[:-1] >= hs[1:])
+
+
+def test_pruned_with_unit_ratios_is_exact(capi, ctx, oracle, blobs):
+    """With every ratio = 1 the bound partial <= full is safe, so the search must equal brute force."""
+    n, d, k = 3000, 256, 1300
+    X, C, prev = _setup(oracle, blobs, n, d, k, seed=77)
+    ratios = np.ones(d + 1, dtype=np.float32)
+    gi, gd, _, _ = _pruned(capi, ctx, oracle, X, C, prev, 32, ratios)
+    bi, bbest, bsecond = oracle.brute_force(X, C)
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    assert np.all((gi == bi) | tie)
+    assert np.allclose(gd, bbest, rtol=1e-4, atol=1e-6)
+
+
+def test_pruned_bad_seed_assignments_still_converge_to_nearest(capi, ctx, oracle, blobs):
+    """Random previous assignments give a loose first threshold (many survivors) but the same answer."""
+    n, d, k = 1500, 256, 1100
+    X, C, _ = _setup(oracle, blobs, n, d, k, seed=5)
+    prev = np.random.default_rng(1).integers(0, k, n).astype(np.uint32)
+    ratios = oracle.ratios(d, 1.5)
+    gi, gd, gtotal, _ = _pruned(capi, ctx, oracle, X, C, prev, 32, ratios)
+    oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, 32, ratios)
+    bi, _, _ = oracle.brute_force(X, C)
+    assert np.mean(gi == oi) >= 0.9999
+    assert np.mean(gi == bi) >= 0.98  # tests/test_assign.cpp:152-155
+    assert abs(int(gtotal) - int(ocounts.sum())) <= max(3, int(1e-2 * ocounts.sum()))
+
+
+def test_pruned_incumbent_only_survivor_keeps_seed_distance(capi, ctx, oracle):
+    """Two far apart centroids: the only survivor is the incumbent, so the seed distance (full
+    Horizontal over d, batch_computers.h:372-377) is returned unchanged (pdxearch.h:140-143)."""
+    d = 128
+    g = np.random.default_rng(2)
+    C = np.zeros((2, d), dtype=np.float32)
+    C[1] += 100.0
+    X = (C[np.array([0, 1, 0, 1])] + 0.01 * g.standard_normal((4, d))).astype(np.float32)
+    prev = np.array([0, 1, 0, 1], dtype=np.uint32)
+    ratios = oracle.ratios(d, 1.5)
+    gi, gd, gtotal, _ = _pruned(capi, ctx, oracle, X, C, prev, 32, ratios)
+    assert np.array_equal(gi, prev)
+    assert gtotal == 4
+    full = ((X.astype(np.float64) - C[prev].astype(np.float64)) ** 2).sum(1)
+    assert np.allclose(gd, full, rtol=1e-5)
