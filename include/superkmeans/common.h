@@ -1,0 +1,154 @@
+// Constants and enums of the Super K-Means public interface, HIP backend.
+// Values follow the reference's include/superkmeans/common.h:89-129; they are part of the
+// algorithm (batch shapes decide tie-breaking and threshold schedules), not tuning knobs.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "skm_hip.h"
+
+#define SKMEANS_ENSURE_POSITIVE(x)                                                                 \
+    if ((x) <= 0) {                                                                                \
+        throw std::invalid_argument("Value must be positive: " #x);                                \
+    }
+
+namespace skmeans {
+
+static inline constexpr float PROPORTION_HORIZONTAL_DIM = 0.75;
+static inline constexpr size_t D_THRESHOLD_FOR_DCT_ROTATION = 512;
+static inline constexpr size_t H_DIM_SIZE = SKM_H_DIM_SIZE;
+static inline constexpr uint32_t MIN_PARTIAL_D = 16;
+static inline constexpr size_t DIMENSION_THRESHOLD_FOR_PRUNING = 128;
+static inline constexpr size_t N_CLUSTERS_THRESHOLD_FOR_PRUNING = 256;
+static inline constexpr size_t X_BATCH_SIZE = SKM_X_BATCH_SIZE;
+static inline constexpr size_t Y_BATCH_SIZE = SKM_Y_BATCH_SIZE;
+static inline constexpr size_t VECTOR_CHUNK_SIZE = Y_BATCH_SIZE;
+static inline constexpr size_t RECALL_CONVERGENCE_PATIENCE = 2;
+static inline constexpr float CENTROID_PERTURBATION_EPS = 1.0f / 1024.0f;
+static inline constexpr float PRUNER_INITIAL_THRESHOLD = 1.5f;
+static inline constexpr float HIERARCHICAL_PRUNER_INITIAL_THRESHOLD = 1.1f;
+
+// Kept for source compatibility: host-side loops of this backend are single threaded, the
+// per-point work runs on the device.
+inline uint32_t g_n_threads = 1;
+
+enum class DistanceFunction : uint8_t { l2, dp };
+enum class Quantization : uint8_t { f32, u8, f16, bf16 };
+
+template <Quantization q>
+struct DistanceType {
+    using type = uint32_t;
+};
+template <>
+struct DistanceType<Quantization::f32> {
+    using type = float;
+};
+template <Quantization q>
+using skmeans_distance_t = typename DistanceType<q>::type;
+
+template <Quantization q>
+struct DataType {
+    using type = uint8_t;
+};
+template <>
+struct DataType<Quantization::f32> {
+    using type = float;
+};
+template <Quantization q>
+using skmeans_value_t = typename DataType<q>::type;
+
+template <Quantization q>
+struct CentroidDataType {
+    using type = float;
+};
+template <Quantization q>
+using skmeans_centroid_value_t = typename CentroidDataType<q>::type;
+
+namespace hip {
+
+// Turns a C-ABI status into the exception type the reference's callers expect.
+inline void Check(int rc) {
+    if (rc == SKM_OK) return;
+    const char* msg = skm_last_error();
+    std::string text = std::string("libskm_hip: ") + (msg ? msg : "unknown error");
+    if (rc == SKM_ERR_INVALID) throw std::invalid_argument(text);
+    throw std::runtime_error(text);
+}
+
+// Owns one skm_ctx (device + stream + workspace).
+class Context {
+  public:
+    explicit Context(int device = 0) { Check(skm_ctx_create(device, &ctx_)); }
+    ~Context() {
+        if (ctx_) skm_ctx_destroy(ctx_);
+    }
+    Context(const Context&) = delete;
+    Context& operator=(const Context&) = delete;
+    skm_ctx* get() const { return ctx_; }
+
+  private:
+    skm_ctx* ctx_ = nullptr;
+};
+
+// A typed device allocation; replaces the std::unique_ptr<T[]> members of the reference.
+template <class T>
+class Buffer {
+  public:
+    Buffer() = default;
+    Buffer(skm_ctx* ctx, size_t count) { Reset(ctx, count); }
+    ~Buffer() { Release(); }
+    Buffer(const Buffer&) = delete;
+    Buffer& operator=(const Buffer&) = delete;
+    Buffer(Buffer&& o) noexcept { MoveFrom(o); }
+    Buffer& operator=(Buffer&& o) noexcept {
+        if (this != &o) {
+            Release();
+            MoveFrom(o);
+        }
+        return *this;
+    }
+    void Reset(skm_ctx* ctx, size_t count) {
+        Release();
+        ctx_ = ctx;
+        count_ = count;
+        void* p = nullptr;
+        Check(skm_malloc(ctx, count * sizeof(T), &p));
+        ptr_ = static_cast<T*>(p);
+    }
+    void Release() {
+        if (ptr_) skm_free(ctx_, ptr_);
+        ptr_ = nullptr;
+        count_ = 0;
+    }
+    T* get() const { return ptr_; }
+    size_t size() const { return count_; }
+    void Upload(const T* host, size_t count, size_t dst_offset = 0) {
+        Check(skm_upload(ctx_, ptr_ + dst_offset, host, count * sizeof(T)));
+    }
+    void Download(T* host, size_t count, size_t src_offset = 0) const {
+        Check(skm_download(ctx_, host, ptr_ + src_offset, count * sizeof(T)));
+    }
+    void swap(Buffer& o) noexcept {
+        std::swap(ctx_, o.ctx_);
+        std::swap(ptr_, o.ptr_);
+        std::swap(count_, o.count_);
+    }
+
+  private:
+    void MoveFrom(Buffer& o) {
+        ctx_ = o.ctx_;
+        ptr_ = o.ptr_;
+        count_ = o.count_;
+        o.ptr_ = nullptr;
+        o.count_ = 0;
+    }
+    skm_ctx* ctx_ = nullptr;
+    T* ptr_ = nullptr;
+    size_t count_ = 0;
+};
+
+} // namespace hip
+} // namespace skmeans

@@ -1,0 +1,326 @@
+// skmeans::HierarchicalSuperKMeans, HIP backend for MI355X.
+//
+// Same public interface as the reference's include/superkmeans/hierarchical_superkmeans.h
+// (config :11-17, stats :22-26, constructors :43-72, Train :84, GetNMesoclusters :549, public
+// members :817-825).  Three phases, all built from SuperKMeans::RunIteration on device buffers:
+//   1. mesoclustering: round(sqrt(k)) clusters over every sample;
+//   2. fine clustering: every mesocluster is gathered into a contiguous device buffer
+//      (skm_gather_rows) and clustered on its own; local ids are scattered back with the running
+//      cluster offset (skm_scatter_assignments);
+//   3. refinement: optional pruned iterations over all k clusters.
+#pragma once
+
+#include "superkmeans/superkmeans.h"
+
+namespace skmeans {
+
+struct HierarchicalSuperKMeansConfig : SuperKMeansConfig {
+    uint32_t iters_mesoclustering = 3;
+    uint32_t iters_fineclustering = 5;
+    uint32_t iters_refinement = 0;
+
+    HierarchicalSuperKMeansConfig() { sampling_fraction = 1.0f; }
+};
+
+struct HierarchicalSuperKMeansIterationStats {
+    std::vector<SuperKMeansIterationStats> mesoclustering_iteration_stats;
+    std::vector<SuperKMeansIterationStats> refinement_iteration_stats;
+    std::vector<SuperKMeansIterationStats> fineclustering_iteration_stats;
+};
+
+template <Quantization q = Quantization::f32, DistanceFunction alpha = DistanceFunction::l2>
+class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
+    using base = SuperKMeans<q, alpha>;
+    using typename base::centroid_value_t;
+    using typename base::vector_value_t;
+    using typename base::pruner_t;
+    using typename base::RowEdit;
+    template <class T>
+    using dbuf = hip::Buffer<T>;
+
+  public:
+    HierarchicalSuperKMeans(size_t n_clusters, size_t dimensionality, const HierarchicalSuperKMeansConfig& config)
+        : base(n_clusters, dimensionality, config), hierarchical_config(config) {
+        // Looser ADSampling epsilon for the hierarchical driver (common.h of the reference, :115).
+        this->pruner = std::make_unique<pruner_t>(this->ctx, dimensionality, HIERARCHICAL_PRUNER_INITIAL_THRESHOLD,
+                                                  this->config.seed);
+        SKMEANS_ENSURE_POSITIVE(config.iters_mesoclustering);
+        SKMEANS_ENSURE_POSITIVE(config.iters_fineclustering);
+        static_cast<SuperKMeansConfig&>(hierarchical_config) = this->config;
+        hierarchical_config.sampling_fraction = config.sampling_fraction;
+        if (n_clusters <= 128 && !this->hierarchical_config.suppress_warnings) {
+            std::cout << "WARNING: n_clusters <= 128 is not recommended for HierarchicalSuperKMeans. "
+                         "Consider using at least 128 clusters."
+                      << std::endl;
+        }
+    }
+
+    HierarchicalSuperKMeans(size_t n_clusters, size_t dimensionality)
+        : HierarchicalSuperKMeans(n_clusters, dimensionality, HierarchicalSuperKMeansConfig{}) {}
+
+    /** Hierarchical training on host-resident data; queries are ignored (as in the reference). */
+    std::vector<centroid_value_t> Train(const vector_value_t* data, const size_t n,
+                                        const vector_value_t* queries = nullptr, const size_t n_queries = 0) {
+        (void) queries;
+        return TrainHierarchical(data, n, n_queries, /*on_device=*/false);
+    }
+
+    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n) {
+        return TrainHierarchical(d_data, n, 0, /*on_device=*/true);
+    }
+
+    static size_t GetNMesoclusters(const size_t n_clusters) {
+        return static_cast<size_t>(std::round(std::sqrt(n_clusters)));
+    }
+
+  protected:
+    std::vector<centroid_value_t> TrainHierarchical(const vector_value_t* data, const size_t n, const size_t n_queries,
+                                                    const bool on_device) {
+        SKMEANS_ENSURE_POSITIVE(n);
+        if (this->trained) {
+            throw std::runtime_error("The clustering has already been trained");
+        }
+        if (n_queries > 0 && !hierarchical_config.suppress_warnings) {
+            std::cout << "WARNING: Early Termination by Recall is not supported in HierarchicalSuperKMeans"
+                      << std::endl;
+        }
+        const size_t k = this->n_clusters;
+        const size_t d = this->d;
+        skm_ctx* ctx = this->ctx;
+        n_mesoclusters = GetNMesoclusters(k);
+        hierarchical_iteration_stats = HierarchicalSuperKMeansIterationStats{};
+        if (n < k) {
+            throw std::runtime_error("The number of points should be at least as large as the number of clusters");
+        }
+        this->n_samples = this->GetNVectorsToSample(n, k);
+        if (this->n_samples < k) {
+            throw std::runtime_error(
+                "Not enough samples to train. Try increasing the sampling_fraction or max_points_per_cluster");
+        }
+        const size_t total_samples = this->n_samples;
+        this->AllocateState(n, k);
+        final_assignments.Reset(ctx, total_samples);
+        final_centroids.Reset(ctx, k * d);
+        this->partial_d = std::max<uint32_t>(MIN_PARTIAL_D, this->vertical_d / 2);
+        if (this->partial_d > this->vertical_d) this->partial_d = this->vertical_d;
+        const uint32_t initial_partial_d = this->partial_d;
+        const bool rotate = !hierarchical_config.data_already_rotated;
+
+        // ---- phase 1: mesoclustering over all samples ----
+        if (hierarchical_config.verbose)
+            std::cout << "\n=== PHASE 1: MESOCLUSTERING (k=" << n_mesoclusters << " clusters) ===" << std::endl;
+        this->GenerateCentroids(data, total_samples, n_mesoclusters, rotate, on_device);
+        const float* data_to_cluster = this->SampleAndRotateVectors(data, n, total_samples, rotate, on_device);
+        this->RotateOrCopy(this->horizontal_centroids.get(), this->prev_centroids.get(), n_mesoclusters, rotate);
+        hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, d, this->data_norms.get()));
+        // Full norms of every sample, kept for the fine phase whose first iteration is always exact.
+        immutable_data_norms.Reset(ctx, total_samples);
+        hip::Check(skm_copy(ctx, immutable_data_norms.get(), this->data_norms.get(), sizeof(float) * total_samples));
+
+        RunPhase(hierarchical_config.iters_mesoclustering, data_to_cluster, total_samples, n_mesoclusters,
+                 hierarchical_config.use_blas_only, /*first_iteration_exact=*/true,
+                 hierarchical_iteration_stats.mesoclustering_iteration_stats, hierarchical_config.early_termination);
+
+        // Sizes as left by the last consolidation, assignments of the last search.
+        mesoclusters_sizes.assign(this->cluster_sizes.get(), this->cluster_sizes.get() + n_mesoclusters);
+        mesoclusters_assignments.resize(total_samples);
+        this->d_assignments.Download(mesoclusters_assignments.data(), total_samples);
+
+        // Point ids grouped by mesocluster, ascending inside each group (counting sort).
+        std::vector<uint64_t> indices_flat(total_samples);
+        std::vector<size_t> offsets(n_mesoclusters + 1, 0);
+        for (size_t m = 0; m < n_mesoclusters; ++m) offsets[m + 1] = offsets[m] + mesoclusters_sizes[m];
+        {
+            std::vector<size_t> cursor(offsets.begin(), offsets.end() - 1);
+            for (size_t i = 0; i < total_samples; ++i) {
+                const size_t m = mesoclusters_assignments[i];
+                if (cursor[m] >= offsets[m + 1]) {
+                    // Sizes were altered by a cluster split in the last mesoclustering iteration and no
+                    // longer describe the assignments; the reference indexes out of range here.
+                    throw std::runtime_error(
+                        "mesocluster sizes are inconsistent with assignments (a mesocluster was split in the "
+                        "last mesoclustering iteration)");
+                }
+                indices_flat[cursor[m]++] = i;
+            }
+        }
+        dbuf<uint64_t> d_indices(ctx, total_samples);
+        d_indices.Upload(indices_flat.data(), total_samples);
+
+        // ---- phase 2: fine clustering, one mesocluster after the other ----
+        if (hierarchical_config.verbose)
+            std::cout << "\n=== PHASE 2: FINE-CLUSTERING (subdividing " << n_mesoclusters << " mesoclusters into total "
+                      << k << " clusters) ===" << std::endl;
+        const auto fine_clusters_nums = ArrangeFineClusters(k, n_mesoclusters, total_samples, mesoclusters_sizes);
+        const size_t max_mesocluster_size = *std::max_element(mesoclusters_sizes.begin(), mesoclusters_sizes.end());
+        dbuf<float> mesocluster_buffer(ctx, std::max<size_t>(1, max_mesocluster_size) * d);
+        size_t fineclusters_offset = 0;
+        for (size_t m = 0; m < n_mesoclusters; ++m) {
+            const size_t n_fineclusters = fine_clusters_nums[m];
+            if (n_fineclusters == 0) continue;
+            this->partial_d = initial_partial_d;
+            const size_t mesocluster_size = mesoclusters_sizes[m];
+            this->n_samples = mesocluster_size;
+            const uint64_t* d_member_ids = d_indices.get() + offsets[m];
+            // Rows and full norms of the members, contiguous (CompactMesoclusterToBuffer).
+            hip::Check(skm_gather_rows(ctx, data_to_cluster, d, d_member_ids, mesocluster_size, mesocluster_buffer.get(),
+                                       immutable_data_norms.get(), this->data_norms.get()));
+            this->GenerateCentroids(mesocluster_buffer.get(), mesocluster_size, n_fineclusters, /*rotate=*/false,
+                                    /*on_device=*/true);
+            hip::Check(skm_copy(ctx, this->prev_centroids.get(), this->horizontal_centroids.get(),
+                                sizeof(float) * n_fineclusters * d));
+            RunPhase(hierarchical_config.iters_fineclustering, mesocluster_buffer.get(), mesocluster_size, n_fineclusters,
+                     hierarchical_config.use_blas_only, /*first_iteration_exact=*/true,
+                     hierarchical_iteration_stats.fineclustering_iteration_stats,
+                     hierarchical_config.early_termination);
+            hip::Check(skm_scatter_assignments(ctx, d_member_ids, this->d_assignments.get(), mesocluster_size,
+                                               static_cast<uint32_t>(fineclusters_offset), final_assignments.get()));
+            hip::Check(skm_copy(ctx, final_centroids.get() + fineclusters_offset * d, this->horizontal_centroids.get(),
+                                sizeof(float) * n_fineclusters * d));
+            fineclusters_offset += n_fineclusters;
+        }
+
+        // ---- phase 3: refinement over all k clusters ----
+        if (hierarchical_config.verbose)
+            std::cout << "\n=== PHASE 3: REFINEMENT (fine-tuning all " << k << " clusters) ===" << std::endl;
+        this->n_samples = total_samples;
+        this->partial_d = std::max<uint32_t>(MIN_PARTIAL_D, this->vertical_d / 3);
+        // SetupCentroids: the concatenated fine centroids become the current centroids in all three
+        // layouts; prev_centroids gets a copy because the next iteration starts with a swap.
+        hip::Check(skm_copy(ctx, this->horizontal_centroids.get(), final_centroids.get(), sizeof(float) * k * d));
+        hip::Check(skm_pdxify(ctx, this->horizontal_centroids.get(), k, d, this->vertical_d, this->centroids.get(),
+                              this->partial_horizontal_centroids.get()));
+        hip::Check(skm_copy(ctx, this->prev_centroids.get(), final_centroids.get(), sizeof(float) * k * d));
+        hip::Check(skm_copy(ctx, this->d_assignments.get(), final_assignments.get(), sizeof(uint32_t) * total_samples));
+        const bool refinement_exact = d < DIMENSION_THRESHOLD_FOR_PRUNING || k <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;
+        bool refinement_norms_ready = false;
+        for (size_t it = 0; it < hierarchical_config.iters_refinement; ++it) {
+            if (!refinement_norms_ready) {
+                // data_norms was reused per mesocluster during phase 2.
+                hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, refinement_exact ? d : this->partial_d,
+                                     this->data_norms.get()));
+                refinement_norms_ready = true;
+            }
+            this->RunIteration(refinement_exact, data_to_cluster, total_samples, k, it, /*is_first_iter=*/false,
+                               hierarchical_iteration_stats.refinement_iteration_stats);
+        }
+        this->trained = true;
+        this->PublishAssignments(total_samples);
+        return this->GetOutputCentroids(hierarchical_config.unrotate_centroids);
+    }
+
+    // Iterations of one phase: the first is always exact (GEMM only); the others are pruned unless the
+    // problem is below the pruning thresholds or use_blas_only is set.
+    void RunPhase(const uint32_t iters, const float* d_points, const size_t n_points, const size_t k_phase,
+                  const bool blas_only, const bool first_iteration_exact, std::vector<SuperKMeansIterationStats>& stats,
+                  const bool early_termination) {
+        const bool always_exact = this->d < DIMENSION_THRESHOLD_FOR_PRUNING || blas_only ||
+                                  k_phase <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;
+        bool partial_norms_computed = false;
+        float best_recall = 0.0f;
+        size_t iters_without_improvement = 0;
+        for (size_t it = 0; it < iters; ++it) {
+            const bool exact = (first_iteration_exact && it == 0) || always_exact;
+            if (!exact && !partial_norms_computed) {
+                hip::Check(skm_norms(this->ctx, d_points, n_points, this->d, this->partial_d, this->data_norms.get()));
+                partial_norms_computed = true;
+            }
+            this->RunIteration(exact, d_points, n_points, k_phase, it, exact && it == 0, stats);
+            if (early_termination && this->ShouldStopEarly(false, best_recall, iters_without_improvement, it)) break;
+        }
+    }
+
+    [[nodiscard]] size_t GetNVectorsToSample(const size_t n, size_t /*n_clusters*/) const override {
+        if (hierarchical_config.sampling_fraction == 1.0) return n;
+        return static_cast<size_t>(std::floor(static_cast<double>(n) * hierarchical_config.sampling_fraction));
+    }
+
+    /**
+     * Empty clusters are re-seeded as in the flat variant; then every cluster smaller than a quarter
+     * of the average size is pulled towards a large cluster chosen with probability proportional to
+     * its excess over the average: c <- (w c + c_large) / (w + 1), w = min(size, 7)
+     * (reference hierarchical_superkmeans.h:579-678).
+     */
+    void SplitClusters(const size_t n_samples_, const size_t k) override {
+        constexpr float CENTER_ADJUSTMENT_WEIGHT = 7.0f;
+        constexpr float BALANCING_THRESHOLD = 0.25f;
+        this->n_split = 0;
+        std::mt19937 rng(this->config.seed);
+        std::vector<RowEdit> edits;
+        auto& sizes = this->cluster_sizes;
+        const size_t average_size = n_samples_ / k;
+        const size_t threshold_size = static_cast<size_t>(static_cast<float>(average_size) * BALANCING_THRESHOLD);
+        for (size_t ci = 0; ci < k; ci++) {
+            if (sizes[ci] != 0) continue;
+            size_t cj;
+            for (cj = 0; true; cj = (cj + 1) % k) {
+                float p = (sizes[cj] - 1.0f) / static_cast<float>(n_samples_ - k);
+                float r = std::uniform_real_distribution<float>(0, 1)(rng);
+                if (r < p) break;
+            }
+            edits.push_back({0u, static_cast<uint32_t>(ci), static_cast<uint32_t>(cj), 0.0f});
+            sizes[ci] = sizes[cj] / 2;
+            sizes[cj] -= sizes[ci];
+            this->n_split++;
+        }
+        for (size_t ci = 0; ci < k; ci++) {
+            const size_t csize = sizes[ci];
+            if (csize == 0 || csize > threshold_size) continue;
+            size_t large;
+            for (large = 0; true; large = (large + 1) % k) {
+                const size_t large_size = sizes[large];
+                if (large_size < average_size) continue;
+                float p = static_cast<float>(large_size - average_size + 1) /
+                          static_cast<float>(n_samples_ - average_size * k + k);
+                float r = std::uniform_real_distribution<float>(0, 1)(rng);
+                if (r < p) break;
+            }
+            const float wc = std::min(static_cast<float>(csize), CENTER_ADJUSTMENT_WEIGHT);
+            edits.push_back({1u, static_cast<uint32_t>(ci), static_cast<uint32_t>(large), wc});
+            this->n_split++;
+        }
+        this->ApplyRowEdits(edits);
+    }
+
+    /**
+     * Fine clusters per mesocluster, proportional to size: lround(remaining_clusters * size /
+     * remaining_samples), at least 1 for a non-empty mesocluster, never so many that a later
+     * non-empty one would get none; the last mesocluster takes what is left
+     * (reference hierarchical_superkmeans.h:718-761).
+     */
+    static std::vector<size_t> ArrangeFineClusters(size_t n_clusters, size_t n_meso, size_t n_samples_,
+                                                   const std::vector<uint32_t>& sizes) {
+        std::vector<size_t> out(n_meso, 0);
+        size_t clusters_left = n_clusters, samples_left = n_samples_;
+        size_t nonempty_left = 0;
+        for (size_t i = 0; i < n_meso; ++i) nonempty_left += sizes[i] > 0 ? 1 : 0;
+        for (size_t i = 0; i < n_meso; ++i) {
+            if (i + 1 == n_meso) {
+                out[i] = clusters_left;
+            } else if (sizes[i] > 0) {
+                nonempty_left--;
+                const double proportion =
+                    static_cast<double>(clusters_left * sizes[i]) / static_cast<double>(samples_left);
+                size_t allocated = static_cast<size_t>(std::lround(proportion));
+                allocated = std::min(allocated, clusters_left - nonempty_left);
+                out[i] = std::max(allocated, size_t{1});
+            }
+            clusters_left -= out[i];
+            samples_left -= sizes[i];
+        }
+        return out;
+    }
+
+    size_t n_mesoclusters = 0;
+    std::vector<uint32_t> mesoclusters_assignments;
+    std::vector<uint32_t> mesoclusters_sizes;
+    dbuf<uint32_t> final_assignments;
+    dbuf<float> immutable_data_norms;
+    dbuf<float> final_centroids;
+
+  public:
+    HierarchicalSuperKMeansConfig hierarchical_config;
+    HierarchicalSuperKMeansIterationStats hierarchical_iteration_stats;
+};
+
+} // namespace skmeans

@@ -1,0 +1,140 @@
+// ADSampling pruner, HIP backend: threshold ratios and the random orthogonal rotation.
+//
+// Mirrors the interface of the reference's ADSamplingPruner (pdx/adsampling.h:29-328, dense-matrix
+// variant): the ratios table, Rotate and Unrotate.  The d x d matrix is built on the host and kept
+// on the device (Q and Q^T); Rotate/Unrotate are MFMA GEMMs (skm_rotate / skm_unrotate).
+#pragma once
+
+#include <cmath>
+#include <random>
+#include <vector>
+
+#include "superkmeans/common.h"
+
+namespace skmeans {
+
+namespace detail {
+
+// Q factor of the Householder QR of `a` (d x d, row-major, double), i.e. H_0 H_1 ... H_{d-1}.
+// Evaluated in double.  Translation units that must reproduce the matrix bit for bit across
+// compilers (the library's own) are built with -ffp-contract=off; otherwise fused multiply-adds may
+// change the last bits of the draws and of the factor, which is harmless for clustering.
+inline std::vector<float> OrthogonalFactor(std::vector<double> a, const size_t d) {
+    std::vector<double> reflectors(d * d, 0.0);  // column j holds reflector j in rows j..d-1
+    std::vector<double> scale(d, 0.0);
+    std::vector<double> w(d);
+    for (size_t j = 0; j < d; ++j) {
+        double norm2 = 0.0;
+        for (size_t r = j; r < d; ++r) {
+            const double v = a[r * d + j];
+            reflectors[r * d + j] = v;
+            norm2 += v * v;
+        }
+        const double norm = std::sqrt(norm2);
+        if (norm == 0.0) continue;
+        const double head = reflectors[j * d + j];
+        const double alpha = (head >= 0.0) ? -norm : norm;
+        reflectors[j * d + j] = head - alpha;
+        double vtv = 0.0;
+        for (size_t r = j; r < d; ++r) vtv += reflectors[r * d + j] * reflectors[r * d + j];
+        if (vtv == 0.0) continue;
+        scale[j] = 2.0 / vtv;
+        for (size_t c = j; c < d; ++c) w[c] = 0.0;
+        for (size_t r = j; r < d; ++r) {
+            const double vr = reflectors[r * d + j];
+            const double* row = &a[r * d];
+            for (size_t c = j; c < d; ++c) w[c] += vr * row[c];
+        }
+        for (size_t r = j; r < d; ++r) {
+            const double f = scale[j] * reflectors[r * d + j];
+            double* row = &a[r * d];
+            for (size_t c = j; c < d; ++c) row[c] -= f * w[c];
+        }
+    }
+    std::vector<double> q(d * d, 0.0);
+    for (size_t i = 0; i < d; ++i) q[i * d + i] = 1.0;
+    for (size_t j = d; j-- > 0;) {
+        if (scale[j] == 0.0) continue;
+        for (size_t c = 0; c < d; ++c) w[c] = 0.0;
+        for (size_t r = j; r < d; ++r) {
+            const double vr = reflectors[r * d + j];
+            const double* row = &q[r * d];
+            for (size_t c = 0; c < d; ++c) w[c] += vr * row[c];
+        }
+        for (size_t r = j; r < d; ++r) {
+            const double f = scale[j] * reflectors[r * d + j];
+            double* row = &q[r * d];
+            for (size_t c = 0; c < d; ++c) row[c] -= f * w[c];
+        }
+    }
+    std::vector<float> out(d * d);
+    for (size_t i = 0; i < d * d; ++i) out[i] = static_cast<float>(q[i]);
+    return out;
+}
+
+} // namespace detail
+
+template <Quantization q = Quantization::f32>
+class ADSamplingPruner {
+  public:
+    uint32_t num_dimensions;
+    std::vector<float> ratios;  // ratios[v]: factor applied to the best distance after v dimensions
+
+    // Draws d*d N(0,1) values row by row from std::mt19937(seed) through
+    // std::normal_distribution<float> (the reference's sequence, pdx/adsampling.h:76-82) and keeps
+    // the orthogonal factor of their QR decomposition.
+    ADSamplingPruner(skm_ctx* ctx, uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42)
+        : num_dimensions(num_dimensions_), ctx_(ctx), epsilon0(epsilon0_) {
+        InitializeRatios();
+        const size_t d = num_dimensions;
+        std::mt19937 gen(seed);
+        std::normal_distribution<float> dist(0.0f, 1.0f);
+        std::vector<double> a(d * d);
+        for (size_t i = 0; i < d * d; ++i) a[i] = dist(gen);
+        matrix_ = detail::OrthogonalFactor(std::move(a), d);
+        d_q_.Reset(ctx_, d * d);
+        d_qt_.Reset(ctx_, d * d);
+        d_q_.Upload(matrix_.data(), d * d);
+        hip::Check(skm_transpose(ctx_, d_q_.get(), d, d, d_qt_.get()));
+    }
+
+    void InitializeRatios() {
+        ratios.resize(num_dimensions + 1);
+        for (size_t v = 0; v <= num_dimensions; ++v) ratios[v] = GetRatio(v);
+        d_ratios_.Reset(ctx_, ratios.size());
+        d_ratios_.Upload(ratios.data(), ratios.size());
+    }
+
+    void SetEpsilon0(float eps0) {
+        epsilon0 = eps0;
+        InitializeRatios();
+    }
+
+    // out = vectors . Q^T, both device-resident (n x d).
+    void Rotate(const float* d_vectors, float* d_out, const size_t n) const {
+        hip::Check(skm_rotate(ctx_, d_vectors, n, num_dimensions, d_q_.get(), d_out));
+    }
+    // out = rotated . Q, both device-resident.
+    void Unrotate(const float* d_rotated, float* d_out, const size_t n) const {
+        hip::Check(skm_unrotate(ctx_, d_rotated, n, num_dimensions, d_qt_.get(), d_out));
+    }
+
+    const float* DeviceRatios() const { return d_ratios_.get(); }
+    const std::vector<float>& HostMatrix() const { return matrix_; }
+
+    // (v / d) * (1 + eps0 / sqrt(v))^2 in double, 1 at v = 0 and v = d (pdx/adsampling.h:315-327).
+    float GetRatio(const size_t visited_dimensions) const {
+        if (visited_dimensions == 0 || visited_dimensions == num_dimensions) return 1.0f;
+        const double v = static_cast<double>(visited_dimensions);
+        const double slack = 1.0 + epsilon0 / std::sqrt(v);
+        return static_cast<float>(v / static_cast<double>(num_dimensions) * slack * slack);
+    }
+
+  private:
+    skm_ctx* ctx_;
+    float epsilon0;
+    std::vector<float> matrix_;
+    hip::Buffer<float> d_q_, d_qt_, d_ratios_;
+};
+
+} // namespace skmeans

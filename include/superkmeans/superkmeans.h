@@ -1,0 +1,720 @@
+// skmeans::SuperKMeans, HIP backend for MI355X.
+//
+// Same public interface as the reference's include/superkmeans/superkmeans.h (config and stats
+// structs :23-98, constructor :123-149, Train :162, Assign :346, AssignTrainingPoints :397,
+// accessors :567-628, public members :1491-1492).  What differs is where the work happens: every
+// per-point step (rotation, norms, distance GEMM, pruned search, centroid update, relayout, cost,
+// shift) is a call into libskm_hip.so on device-resident buffers; this header only keeps the
+// iteration control flow, the RNG-dependent host decisions (initial centroids, sampling, cluster
+// splitting, d' tuning, early stopping) and the transfers at the API boundary.
+//
+// Additions over the reference interface (they do not change existing calls):
+//   TrainDevice / AssignDevice   same as Train / Assign for inputs that already live in HBM.
+//   GetContext                   the skm_ctx used by this object (device timers, workspace limit).
+#pragma once
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <iostream>
+#include <memory>
+#include <numeric>
+#include <random>
+#include <sstream>
+#include <vector>
+
+#include "superkmeans/common.h"
+#include "superkmeans/pdx/adsampling.h"
+#include "superkmeans/pdx/layout.h"
+
+namespace skmeans {
+
+struct SuperKMeansConfig {
+    // Training parameters
+    uint32_t iters = 10;
+    float sampling_fraction = 0.3f;
+    uint32_t max_points_per_cluster = 256;
+    uint32_t n_threads = 0;  // accepted for compatibility; device work does not use host threads
+    uint32_t seed = 42;
+    bool use_blas_only = false;  // GEMM-only iterations (no pruning)
+
+    // Convergence parameters
+    float tol = 1e-4f;
+    float recall_tol = 0.005f;
+    bool early_termination = true;
+    bool sample_queries = false;
+    size_t objective_k = 100;
+    float ann_explore_fraction = 0.01f;
+
+    // Sweet range for d' tuning
+    float min_not_pruned_pct = 0.03f;
+    float max_not_pruned_pct = 0.05f;
+    float adjustment_factor_for_partial_d = 0.20f;
+
+    // Output parameters
+    bool unrotate_centroids = true;
+    bool verbose = false;
+    bool angular = false;
+    bool suppress_warnings = false;
+
+    bool data_already_rotated = false;
+};
+
+struct SuperKMeansIterationStats {
+    size_t iteration = 0;
+    float objective = 0.0f;
+    float shift = 0.0f;
+    size_t split = 0;
+    float recall = 0.0f;
+    float not_pruned_pct = -1.0f;
+    uint32_t partial_d = 0;
+    bool is_gemm_only = false;
+};
+
+struct ClusterBalanceStats {
+    float mean = 0.0f;
+    float geometric_mean = 0.0f;
+    float stdev = 0.0f;
+    float cv = 0.0f;
+    size_t min = 0;
+    size_t max = 0;
+
+    std::string to_json() const {
+        std::ostringstream oss;
+        oss << "{\"mean\":" << mean << ",\"geometric_mean\":" << geometric_mean << ",\"stdev\":" << stdev
+            << ",\"cv\":" << cv << ",\"min\":" << min << ",\"max\":" << max << "}";
+        return oss.str();
+    }
+
+    void print() const {
+        std::cout << "Cluster size stats: mean=" << mean << ", gmean=" << geometric_mean << ", std=" << stdev
+                  << ", CV=" << cv << ", min=" << min << ", max=" << max << std::endl;
+    }
+};
+
+template <Quantization q = Quantization::f32, DistanceFunction alpha = DistanceFunction::l2>
+class SuperKMeans {
+    static_assert(q == Quantization::f32 && alpha == DistanceFunction::l2,
+                  "only <f32, l2> is instantiated, as in the reference");
+
+  public:
+    virtual ~SuperKMeans() = default;
+
+  protected:
+    using centroid_value_t = skmeans_centroid_value_t<q>;
+    using vector_value_t = skmeans_value_t<q>;
+    using distance_t = skmeans_distance_t<q>;
+    using pruner_t = ADSamplingPruner<q>;
+    using layout_t = PDXLayout<q, alpha>;
+    template <class T>
+    using dbuf = hip::Buffer<T>;
+
+  public:
+    SuperKMeans(size_t n_clusters, size_t dimensionality, const SuperKMeansConfig& config)
+        : d(dimensionality), n_clusters(n_clusters), config(config) {
+        SKMEANS_ENSURE_POSITIVE(n_clusters);
+        SKMEANS_ENSURE_POSITIVE(dimensionality);
+        SKMEANS_ENSURE_POSITIVE(config.iters);
+        SKMEANS_ENSURE_POSITIVE(config.sampling_fraction);
+        if (config.sampling_fraction > 1.0) {
+            throw std::invalid_argument("sampling_fraction must be <= 1.0");
+        }
+        n_threads = (config.n_threads == 0) ? 1 : config.n_threads;
+        g_n_threads = n_threads;
+        context = std::make_shared<hip::Context>(0);
+        ctx = context->get();
+        pruner = std::make_unique<pruner_t>(ctx, dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed);
+        if (this->config.data_already_rotated) {
+            this->config.unrotate_centroids = false;
+        }
+    }
+
+    SuperKMeans(size_t n_clusters, size_t dimensionality)
+        : SuperKMeans(n_clusters, dimensionality, SuperKMeansConfig{}) {}
+
+    /** Runs k-means on host-resident row-major data (n x d) and returns the k x d centroids. */
+    std::vector<centroid_value_t> Train(const vector_value_t* data, const size_t n,
+                                        const vector_value_t* queries = nullptr, const size_t n_queries = 0) {
+        return TrainImpl(data, n, queries, n_queries, /*on_device=*/false);
+    }
+
+    /** Train for data that already lives in device memory of this object's context. */
+    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n) {
+        return TrainImpl(d_data, n, nullptr, 0, /*on_device=*/true);
+    }
+
+    /** Exact nearest-centroid assignment; vectors and centroids must be in the same space. */
+    [[nodiscard]] std::vector<uint32_t> Assign(const vector_value_t* vectors, const vector_value_t* centroids,
+                                               const size_t n_vectors, const size_t n_centroids) {
+        dbuf<float> d_v(ctx, n_vectors * d), d_c(ctx, n_centroids * d);
+        d_v.Upload(vectors, n_vectors * d);
+        d_c.Upload(centroids, n_centroids * d);
+        dbuf<uint32_t> d_out(ctx, n_vectors);
+        AssignDevice(d_v.get(), d_c.get(), n_vectors, n_centroids, d_out.get());
+        std::vector<uint32_t> result(n_vectors);
+        d_out.Download(result.data(), n_vectors);
+        return result;
+    }
+
+    /** Assign on device-resident inputs; writes n_vectors indices to d_out_assignments (asynchronous). */
+    void AssignDevice(const vector_value_t* d_vectors, const vector_value_t* d_centroids, const size_t n_vectors,
+                      const size_t n_centroids, uint32_t* d_out_assignments) {
+        dbuf<float> v_norms(ctx, n_vectors), c_norms(ctx, n_centroids), dist(ctx, n_vectors);
+        hip::Check(skm_norms(ctx, d_vectors, n_vectors, d, d, v_norms.get()));
+        hip::Check(skm_norms(ctx, d_centroids, n_centroids, d, d, c_norms.get()));
+        hip::Check(skm_assign_full(ctx, d_vectors, n_vectors, d_centroids, n_centroids, d, v_norms.get(),
+                                   c_norms.get(), d_out_assignments, dist.get()));
+        hip::Check(skm_sync(ctx));  // the scratch buffers above are released on return
+    }
+
+    /** Pruned assignment of the training points, seeded with the assignments found by Train. */
+    [[nodiscard]] std::vector<uint32_t> AssignTrainingPoints(const vector_value_t* vectors,
+                                                             const vector_value_t* centroids,
+                                                             const size_t n_vectors, const size_t n_centroids) {
+        if (!trained) {
+            throw std::runtime_error("AssignTrainingPoints requires SuperKMeans to be trained first");
+        }
+        if (config.use_blas_only || d < DIMENSION_THRESHOLD_FOR_PRUNING ||
+            n_clusters <= N_CLUSTERS_THRESHOLD_FOR_PRUNING) {
+            if (!config.suppress_warnings) {
+                std::cout << "WARNING: AssignTrainingPoints cannot use pruning, falling back to "
+                             "brute force Assign"
+                          << std::endl;
+            }
+            return Assign(vectors, centroids, n_vectors, n_centroids);
+        }
+        partial_d = std::max<uint32_t>(MIN_PARTIAL_D, vertical_d / 2);
+
+        // Rotated copy of the caller's vectors (or the vectors themselves when already rotated).
+        dbuf<float> d_rot(ctx, n_vectors * d);
+        {
+            if (config.data_already_rotated) {
+                d_rot.Upload(vectors, n_vectors * d);
+            } else {
+                dbuf<float> d_raw(ctx, n_vectors * d);
+                d_raw.Upload(vectors, n_vectors * d);
+                pruner->Rotate(d_raw.get(), d_rot.get(), n_vectors);
+                hip::Check(skm_sync(ctx));
+            }
+        }
+        // Final centroids: horizontal_centroids / centroids (PDX) / partial_horizontal_centroids were
+        // all refreshed by the last ConsolidateCentroids.
+        hip::Check(skm_norms(ctx, horizontal_centroids.get(), n_centroids, d, partial_d, centroid_norms.get()));
+
+        std::vector<uint32_t> seeds(n_vectors);
+        if (config.sampling_fraction == 1.0f) {
+            std::memcpy(seeds.data(), assignments.get(), n_vectors * sizeof(uint32_t));
+        } else if (config.sampling_fraction > 0.8f) {
+            // Sampled points keep their training assignment, the rest draw a cluster with
+            // probability proportional to its size.
+            size_t cur = 0;
+            for (; cur < n_samples; ++cur) seeds[sampled_indices[cur]] = assignments[cur];
+            std::mt19937 rng(config.seed + 1);
+            std::discrete_distribution<uint32_t> cluster_dist(cluster_sizes.get(), cluster_sizes.get() + n_clusters);
+            for (; cur < n_vectors; ++cur) seeds[sampled_indices[cur]] = cluster_dist(rng);
+        } else {
+            // Few samples: cluster the centroids into sqrt(k) meso-centroids and seed every
+            // unsampled point with a representative of its nearest meso-centroid.
+            SuperKMeansConfig tmp_config;
+            tmp_config.iters = 10;
+            tmp_config.sampling_fraction = 1.0f;
+            tmp_config.use_blas_only = false;
+            tmp_config.verbose = config.verbose;
+            tmp_config.suppress_warnings = config.suppress_warnings;
+            tmp_config.seed = config.seed;
+            tmp_config.angular = config.angular;
+            tmp_config.data_already_rotated = config.data_already_rotated;
+            auto new_n_centroids = static_cast<size_t>(std::sqrt(n_centroids));
+            SuperKMeans tmp_kmeans(new_n_centroids, d, tmp_config);
+            auto meso_centroids = tmp_kmeans.Train(centroids, n_centroids);
+            auto meso_assignments = tmp_kmeans.Assign(vectors, meso_centroids.data(), n_vectors, new_n_centroids);
+            auto centroids_to_meso = tmp_kmeans.Assign(centroids, meso_centroids.data(), n_centroids, new_n_centroids);
+            g_n_threads = n_threads;
+            std::vector<uint32_t> meso_to_original(new_n_centroids, 0);
+            for (size_t c = 0; c < n_centroids; ++c) meso_to_original[centroids_to_meso[c]] = static_cast<uint32_t>(c);
+            size_t cur = 0;
+            for (; cur < n_samples; ++cur) seeds[sampled_indices[cur]] = assignments[cur];
+            for (; cur < n_vectors; ++cur) {
+                const size_t orig_idx = sampled_indices[cur];
+                seeds[orig_idx] = meso_to_original[meso_assignments[orig_idx]];
+            }
+        }
+        dbuf<uint32_t> d_seed(ctx, n_vectors);
+        d_seed.Upload(seeds.data(), n_vectors);
+        dbuf<float> d_norms_p(ctx, n_vectors), d_dist(ctx, n_vectors);
+        hip::Check(skm_norms(ctx, d_rot.get(), n_vectors, d, partial_d, d_norms_p.get()));
+        uint64_t not_pruned_total = 0;
+        hip::Check(skm_assign_pruned(ctx, d_rot.get(), n_vectors, horizontal_centroids.get(), this->centroids.get(),
+                                     partial_horizontal_centroids.get(), n_clusters, d, vertical_d, partial_d,
+                                     pruner->DeviceRatios(), d_norms_p.get(), centroid_norms.get(), d_seed.get(),
+                                     d_dist.get(), &not_pruned_total, nullptr));
+        std::vector<uint32_t> result(n_vectors);
+        d_seed.Download(result.data(), n_vectors);
+        if (config.sampling_fraction == 1.0f) {
+            // The reference updates the object's assignments/distances in this branch (:454-469).
+            std::memcpy(assignments.get(), result.data(), n_vectors * sizeof(uint32_t));
+            host_distances.resize(n_vectors);
+            d_dist.Download(host_distances.data(), n_vectors);
+        }
+        return result;
+    }
+
+    [[nodiscard]] size_t GetNClusters() const noexcept { return n_clusters; }
+    [[nodiscard]] bool IsTrained() const noexcept { return trained; }
+    [[nodiscard]] float GetSamplingFraction() const noexcept { return config.sampling_fraction; }
+    /** Host copy of the per-point squared distances of the last training iteration. */
+    [[nodiscard]] distance_t* GetDistancesPointer() { return host_distances.data(); }
+    [[nodiscard]] skm_ctx* GetContext() const noexcept { return ctx; }
+
+    [[nodiscard]] static ClusterBalanceStats GetClustersBalanceStats(const uint32_t* assignments_in, size_t n_samples_in,
+                                                                     size_t n_clusters_in) {
+        ClusterBalanceStats stats;
+        std::vector<size_t> sizes(n_clusters_in, 0);
+        for (size_t i = 0; i < n_samples_in; ++i) sizes[assignments_in[i]]++;
+        const auto sum = std::accumulate(sizes.begin(), sizes.end(), size_t{0});
+        stats.mean = static_cast<float>(sum) / static_cast<float>(sizes.size());
+        float log_sum = 0.0f;
+        size_t non_zero = 0;
+        size_t sq_sum = 0;
+        for (size_t s : sizes) {
+            if (s > 0) {
+                log_sum += std::log(static_cast<float>(s));
+                non_zero++;
+            }
+            sq_sum += s * s;
+        }
+        stats.geometric_mean = non_zero > 0 ? std::exp(log_sum / static_cast<float>(non_zero)) : 0.0f;
+        stats.stdev = std::sqrt(static_cast<float>(sq_sum) / static_cast<float>(sizes.size()) - stats.mean * stats.mean);
+        stats.cv = stats.stdev / stats.mean;
+        const auto mm = std::minmax_element(sizes.begin(), sizes.end());
+        stats.min = *mm.first;
+        stats.max = *mm.second;
+        return stats;
+    }
+
+  protected:
+    // ------------------------------------------------------------------------------------------
+    // Train, flat variant (reference superkmeans.h:162-332)
+    // ------------------------------------------------------------------------------------------
+    std::vector<centroid_value_t> TrainImpl(const vector_value_t* data, const size_t n, const vector_value_t* queries,
+                                            const size_t n_queries, const bool on_device) {
+        SKMEANS_ENSURE_POSITIVE(n);
+        if (trained) {
+            throw std::runtime_error("The clustering has already been trained");
+        }
+        iteration_stats.clear();
+        if (n < n_clusters) {
+            throw std::runtime_error("The number of points should be at least as large as the number of clusters");
+        }
+        if (n_queries > 0 && queries == nullptr && !config.sample_queries) {
+            throw std::invalid_argument("Queries must be provided if n_queries > 0 and sample_queries is false");
+        }
+        if (n_queries > 0) {
+            throw std::runtime_error(
+                "recall-based early termination (queries) is not available in the HIP backend yet");
+        }
+        n_samples = GetNVectorsToSample(n, n_clusters);
+        if (n_samples < n_clusters) {
+            throw std::runtime_error(
+                "Not enough samples to train. Try increasing the sampling_fraction or max_points_per_cluster");
+        }
+        AllocateState(n, n_clusters);
+        partial_d = std::max<uint32_t>(MIN_PARTIAL_D, vertical_d / 2);
+        if (partial_d > vertical_d) partial_d = vertical_d;
+        if (config.verbose) {
+            std::cout << "Front dimensions (d') = " << partial_d << std::endl;
+            std::cout << "Trailing dimensions (d'') = " << d - vertical_d << std::endl;
+        }
+
+        const bool rotate = !config.data_already_rotated;
+        GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
+        const float* data_to_cluster = SampleAndRotateVectors(data, n, n_samples, rotate, on_device);
+        // prev_centroids <- rotated initial centroids; horizontal_centroids still holds the raw rows.
+        RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
+        hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, d, data_norms.get()));
+
+        const bool always_gemm_only = d < DIMENSION_THRESHOLD_FOR_PRUNING || config.use_blas_only ||
+                                      n_clusters <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;
+        bool partial_norms_computed = false;
+        float best_recall = 0.0f;
+        size_t iters_without_improvement = 0;
+        for (size_t iter_idx = 0; iter_idx < config.iters; ++iter_idx) {
+            const bool use_gemm_only = (iter_idx == 0) || always_gemm_only;
+            if (!use_gemm_only && !partial_norms_computed) {
+                hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, partial_d, data_norms.get()));
+                partial_norms_computed = true;
+            }
+            RunIteration(use_gemm_only, data_to_cluster, n_samples, n_clusters, iter_idx,
+                         use_gemm_only && iter_idx == 0, iteration_stats);
+            if (config.early_termination && ShouldStopEarly(false, best_recall, iters_without_improvement, iter_idx)) {
+                break;
+            }
+        }
+        trained = true;
+        PublishAssignments(n_samples);
+        return GetOutputCentroids(config.unrotate_centroids);
+    }
+
+    // Device and host state sized like the reference's buffers (superkmeans.h:191-209).
+    void AllocateState(const size_t n, const size_t k) {
+        vertical_d = static_cast<uint32_t>(layout_t::GetDimensionSplit(d).vertical_d);
+        centroids.Reset(ctx, k * d);
+        horizontal_centroids.Reset(ctx, k * d);
+        prev_centroids.Reset(ctx, k * d);
+        partial_horizontal_centroids.Reset(ctx, k * vertical_d);
+        d_cluster_sizes.Reset(ctx, k);
+        d_assignments.Reset(ctx, n);
+        distances.Reset(ctx, n);
+        data_norms.Reset(ctx, n_samples);
+        centroid_norms.Reset(ctx, k);
+        cluster_sizes.reset(new uint32_t[k]);
+        assignments.reset(new uint32_t[n]);
+    }
+
+    // One k-means iteration (reference RunIteration<GEMM_ONLY>, superkmeans.h:786-879).
+    void RunIteration(const bool gemm_only, const float* data_to_cluster, const size_t n_samples_, const size_t k,
+                      const size_t iter_idx, const bool is_first_iter,
+                      std::vector<SuperKMeansIterationStats>& target_stats) {
+        if (!is_first_iter) horizontal_centroids.swap(prev_centroids);
+        uint64_t not_pruned_total = 0;
+        if (gemm_only) {
+            hip::Check(skm_norms(ctx, prev_centroids.get(), k, d, d, centroid_norms.get()));
+            hip::Check(skm_assign_full(ctx, data_to_cluster, n_samples_, prev_centroids.get(), k, d, data_norms.get(),
+                                       centroid_norms.get(), d_assignments.get(), distances.get()));
+        } else {
+            hip::Check(skm_norms(ctx, prev_centroids.get(), k, d, partial_d, centroid_norms.get()));
+            hip::Check(skm_assign_pruned(ctx, data_to_cluster, n_samples_, prev_centroids.get(), centroids.get(),
+                                         partial_horizontal_centroids.get(), k, d, vertical_d, partial_d,
+                                         pruner->DeviceRatios(), data_norms.get(), centroid_norms.get(),
+                                         d_assignments.get(), distances.get(), &not_pruned_total, nullptr));
+        }
+        // Sums and counts (zero-filled by the kernel itself for empty clusters).
+        hip::Check(skm_update(ctx, data_to_cluster, n_samples_, d, d_assignments.get(), k, horizontal_centroids.get(),
+                              d_cluster_sizes.get()));
+
+        float avg_not_pruned_pct = -1.0f;
+        const uint32_t old_partial_d = partial_d;
+        if (!gemm_only) {
+            bool partial_d_changed = false;
+            avg_not_pruned_pct = TunePartialD(not_pruned_total, n_samples_, k, partial_d_changed);
+            if (partial_d_changed) {
+                hip::Check(skm_norms(ctx, data_to_cluster, n_samples_, d, partial_d, data_norms.get()));
+            }
+        }
+        ConsolidateCentroids(n_samples_, k);
+        ComputeCost(n_samples_);
+        ComputeShift(k);
+
+        SuperKMeansIterationStats stats;
+        stats.iteration = iter_idx + 1;
+        stats.objective = cost;
+        stats.shift = shift;
+        stats.split = n_split;
+        stats.recall = recall;
+        stats.is_gemm_only = gemm_only;
+        if (!gemm_only) {
+            stats.not_pruned_pct = avg_not_pruned_pct;
+            stats.partial_d = old_partial_d;
+        }
+        target_stats.push_back(stats);
+        if (config.verbose) {
+            std::cout << "Iteration " << iter_idx + 1 << "/" << config.iters << " | Objective: " << cost
+                      << " | Objective improvement: " << (iter_idx > 0 ? 1 - (cost / prev_cost) : 0.0f)
+                      << " | Shift: " << shift << " | Split: " << n_split << " | Recall: " << recall;
+            if (gemm_only) {
+                std::cout << " [GEMM-only]";
+            } else {
+                std::cout << " | Not Pruned %: " << avg_not_pruned_pct * 100.0f << " | d': " << old_partial_d << " -> "
+                          << partial_d;
+            }
+            std::cout << std::endl << std::endl;
+        }
+    }
+
+    // A pending row edit for skm_edit_rows.
+    struct RowEdit {
+        uint32_t kind, dst, src;
+        float weight;
+    };
+    void ApplyRowEdits(const std::vector<RowEdit>& edits) {
+        if (edits.empty()) return;
+        std::vector<uint32_t> ops(edits.size() * 4);
+        for (size_t i = 0; i < edits.size(); ++i) {
+            ops[4 * i] = edits[i].kind;
+            ops[4 * i + 1] = edits[i].dst;
+            ops[4 * i + 2] = edits[i].src;
+            std::memcpy(&ops[4 * i + 3], &edits[i].weight, sizeof(float));
+        }
+        hip::Check(skm_edit_rows(ctx, horizontal_centroids.get(), d, ops.data(), edits.size()));
+    }
+
+    /**
+     * Empty clusters are re-seeded from a large one (FAISS rule; reference superkmeans.h:890-928):
+     * walk the clusters cyclically and accept cj with probability (size_cj - 1) / (n - k), one
+     * uniform draw from mt19937(seed) per visit; the donor row is copied and both copies perturbed by
+     * (1 +/- 1/1024) alternating per column; the donor's size is split in two.  Decisions need only
+     * the sizes, so they are taken on the host and the row arithmetic is queued for the device.
+     */
+    virtual void SplitClusters(const size_t n_samples_, const size_t k) {
+        n_split = 0;
+        std::mt19937 rng(config.seed);
+        std::vector<RowEdit> edits;
+        for (size_t ci = 0; ci < k; ci++) {
+            if (cluster_sizes[ci] != 0) continue;
+            size_t cj;
+            for (cj = 0; true; cj = (cj + 1) % k) {
+                float p = (cluster_sizes[cj] - 1.0) / (float) (n_samples_ - k);
+                float r = std::uniform_real_distribution<float>(0, 1)(rng);
+                if (r < p) break;
+            }
+            edits.push_back({0u, static_cast<uint32_t>(ci), static_cast<uint32_t>(cj), 0.0f});
+            cluster_sizes[ci] = cluster_sizes[cj] / 2;
+            cluster_sizes[cj] -= cluster_sizes[ci];
+            n_split++;
+        }
+        ApplyRowEdits(edits);
+    }
+
+    // Means, empty-cluster handling, optional normalisation, PDX relayout (superkmeans.h:936-968).
+    void ConsolidateCentroids(const size_t n_samples_, const size_t k) {
+        hip::Check(skm_scale_by_size(ctx, horizontal_centroids.get(), d_cluster_sizes.get(), k, d));
+        d_cluster_sizes.Download(cluster_sizes.get(), k);
+        SplitClusters(n_samples_, k);
+        if (config.angular) {
+            hip::Check(skm_normalize_rows(ctx, horizontal_centroids.get(), k, d));
+        }
+        hip::Check(skm_pdxify(ctx, horizontal_centroids.get(), k, d, vertical_d, centroids.get(),
+                              partial_horizontal_centroids.get()));
+    }
+
+    // WCSS of this iteration's assignments; accumulated in fp64 on the device (superkmeans.h:973-981
+    // sums the same values in fp32).
+    void ComputeCost(const size_t n_samples_) {
+        prev_cost = cost;
+        double c = 0.0;
+        hip::Check(skm_wcss(ctx, distances.get(), n_samples_, &c));
+        cost_f64 = c;
+        cost = static_cast<float>(c);
+    }
+
+    void ComputeShift(const size_t k) {
+        double s = 0.0;
+        hip::Check(skm_shift(ctx, horizontal_centroids.get(), prev_centroids.get(), k, d, &s));
+        shift = static_cast<float>(s);
+    }
+
+    /**
+     * Forgy initialisation (reference superkmeans.h:1100-1142): shuffle [0, n_points) with
+     * mt19937(seed) and take the first k rows of `data`; the rows land in horizontal_centroids
+     * (raw) and their rotated, PDX-laid-out copy in `centroids`.
+     */
+    void GenerateCentroids(const vector_value_t* data, const size_t n_points, const size_t k, const bool rotate,
+                           const bool on_device) {
+        if (k > n_points) {
+            throw std::runtime_error("cannot draw more initial centroids than there are points");
+        }
+        std::mt19937 rng(config.seed);
+        std::vector<size_t> indices(n_points);
+        std::iota(indices.begin(), indices.end(), size_t{0});
+        std::shuffle(indices.begin(), indices.end(), rng);
+        if (on_device) {
+            std::vector<uint64_t> rows(indices.begin(), indices.begin() + k);
+            dbuf<uint64_t> d_rows(ctx, k);
+            d_rows.Upload(rows.data(), k);
+            hip::Check(skm_gather_rows(ctx, data, d, d_rows.get(), k, horizontal_centroids.get(), nullptr, nullptr));
+            hip::Check(skm_sync(ctx));
+        } else {
+            std::vector<float> staged(k * d);
+            for (size_t i = 0; i < k; ++i) std::memcpy(&staged[i * d], data + indices[i] * d, sizeof(float) * d);
+            horizontal_centroids.Upload(staged.data(), k * d);
+        }
+        dbuf<float> rotated(ctx, k * d);
+        RotateOrCopy(horizontal_centroids.get(), rotated.get(), k, rotate);
+        hip::Check(skm_pdxify(ctx, rotated.get(), k, d, vertical_d, centroids.get(), nullptr));
+        hip::Check(skm_sync(ctx));
+    }
+
+    void RotateOrCopy(const float* d_in, float* d_out, const size_t n_vectors, const bool rotate) {
+        if (rotate) {
+            pruner->Rotate(d_in, d_out, n_vectors);
+        } else {
+            hip::Check(skm_copy(ctx, d_out, d_in, sizeof(float) * n_vectors * d));
+        }
+    }
+
+    /**
+     * d' tuning (reference superkmeans.h:1230-1258): p = not-pruned pairs / (n * k); above
+     * max_not_pruned_pct grow d' by 2 * adjustment (at least 1) up to vertical_d, below
+     * min_not_pruned_pct shrink it by adjustment (at least 1) down to MIN_PARTIAL_D.  The pair count
+     * is summed exactly on the device.
+     */
+    float TunePartialD(const uint64_t not_pruned_total, size_t n_samples_, size_t n_y, bool& partial_d_changed) {
+        float avg_not_pruned_pct = static_cast<float>(static_cast<double>(not_pruned_total));
+        avg_not_pruned_pct /= static_cast<float>(n_samples_ * n_y);
+        const uint32_t old_partial_d = partial_d;
+        if (avg_not_pruned_pct > config.max_not_pruned_pct) {
+            auto increase = static_cast<uint32_t>(partial_d * config.adjustment_factor_for_partial_d * 2);
+            partial_d = std::min(partial_d + std::max(increase, 1u), vertical_d);
+        } else if (avg_not_pruned_pct < config.min_not_pruned_pct) {
+            auto decrease = static_cast<uint32_t>(partial_d * config.adjustment_factor_for_partial_d);
+            partial_d = std::max(partial_d - std::max(decrease, 1u), MIN_PARTIAL_D);
+        }
+        partial_d_changed = (old_partial_d != partial_d);
+        return avg_not_pruned_pct;
+    }
+
+    [[nodiscard]] virtual size_t GetNVectorsToSample(const size_t n, size_t k) const {
+        if (config.sampling_fraction == 1.0) return n;
+        auto samples_by_clusters = k * config.max_points_per_cluster;
+        auto samples_by_n = static_cast<size_t>(std::floor(static_cast<float>(n) * config.sampling_fraction));
+        return std::min<size_t>(samples_by_n, samples_by_clusters);
+    }
+
+    bool ShouldStopEarly(const bool tracking_recall, float& best_recall, size_t& iters_without_improvement,
+                         const size_t iter_idx) {
+        if (shift < config.tol) {
+            if (config.verbose)
+                std::cout << "Converged at iteration " << iter_idx + 1 << " (shift " << shift << " < tol "
+                          << config.tol << ")" << std::endl;
+            return true;
+        }
+        if (iter_idx > 0) {
+            auto cost_delta = cost / prev_cost;
+            if (cost_delta > 1 - config.tol) {
+                if (config.verbose)
+                    std::cout << "Converged at iteration " << iter_idx + 1 << " (cost improved by only "
+                              << 1 - cost_delta << ")" << std::endl;
+                return true;
+            }
+        }
+        if (tracking_recall) {
+            float improvement = recall - best_recall;
+            if (improvement > config.recall_tol) {
+                best_recall = recall;
+                iters_without_improvement = 0;
+            } else {
+                iters_without_improvement++;
+                if (iters_without_improvement >= RECALL_CONVERGENCE_PATIENCE) return true;
+            }
+        }
+        return false;
+    }
+
+    std::vector<centroid_value_t> GetOutputCentroids(bool should_unrotate) {
+        std::vector<centroid_value_t> out(n_clusters * d);
+        if (should_unrotate) {
+            dbuf<float> unrotated(ctx, n_clusters * d);
+            pruner->Unrotate(horizontal_centroids.get(), unrotated.get(), n_clusters);
+            unrotated.Download(out.data(), n_clusters * d);
+        } else {
+            horizontal_centroids.Download(out.data(), n_clusters * d);
+        }
+        return out;
+    }
+
+    /**
+     * Produces the (sampled, rotated) training matrix on the device and returns its address
+     * (reference superkmeans.h:1385-1443).  Sampling shuffles [0, n) with mt19937(seed) and takes the
+     * first n_samples indices.  Without rotation and without sampling a device-resident input is
+     * used in place.
+     */
+    const float* SampleAndRotateVectors(const vector_value_t* data, const size_t n, const size_t n_samples_,
+                                        const bool rotate, const bool on_device) {
+        const bool sample = n_samples_ < n;
+        if (sample) {
+            std::mt19937 rng(config.seed);
+            sampled_indices.reset(new size_t[n]);
+            for (size_t i = 0; i < n; ++i) sampled_indices[i] = i;
+            std::shuffle(sampled_indices.get(), sampled_indices.get() + n, rng);
+        }
+        if (on_device && !sample && !rotate) return data;
+        dbuf<float> staged;  // raw rows on the device, in training order
+        const float* d_raw = nullptr;
+        if (on_device && !sample) {
+            d_raw = data;
+        } else if (on_device) {
+            std::vector<uint64_t> rows(sampled_indices.get(), sampled_indices.get() + n_samples_);
+            dbuf<uint64_t> d_rows(ctx, n_samples_);
+            d_rows.Upload(rows.data(), n_samples_);
+            staged.Reset(ctx, n_samples_ * d);
+            hip::Check(skm_gather_rows(ctx, data, d, d_rows.get(), n_samples_, staged.get(), nullptr, nullptr));
+            hip::Check(skm_sync(ctx));
+            d_raw = staged.get();
+        } else {
+            staged.Reset(ctx, n_samples_ * d);
+            if (!sample) {
+                staged.Upload(data, n_samples_ * d);
+            } else {
+                // Gather on the host in slabs so the staging buffer stays small.
+                const size_t slab = std::max<size_t>(1, (size_t(64) << 20) / (d * sizeof(float)));
+                std::vector<float> host(std::min(slab, n_samples_) * d);
+                for (size_t i0 = 0; i0 < n_samples_; i0 += slab) {
+                    const size_t m = std::min(slab, n_samples_ - i0);
+                    for (size_t i = 0; i < m; ++i)
+                        std::memcpy(&host[i * d], data + sampled_indices[i0 + i] * d, sizeof(float) * d);
+                    staged.Upload(host.data(), m * d, i0 * d);
+                }
+            }
+            d_raw = staged.get();
+        }
+        if (!rotate) {
+            training_data = std::move(staged);
+            return training_data.get();
+        }
+        training_data.Reset(ctx, n_samples_ * d);
+        pruner->Rotate(d_raw, training_data.get(), n_samples_);
+        hip::Check(skm_sync(ctx));  // `staged` is released on return
+        return training_data.get();
+    }
+
+    // Copies the device assignments / distances of the training points to the public host members.
+    void PublishAssignments(const size_t count) {
+        d_assignments.Download(assignments.get(), count);
+        host_distances.resize(count);
+        distances.Download(host_distances.data(), count);
+    }
+
+    const size_t d;
+    const size_t n_clusters;
+    SuperKMeansConfig config;
+
+    uint32_t n_threads;
+    size_t n_samples = 0;
+    uint32_t partial_d = 0;
+
+    bool trained = false;
+    size_t n_split = 0;
+    uint32_t vertical_d = 0;
+    float prev_cost = 0.0f;
+    float cost = 0.0f;
+    double cost_f64 = 0.0;
+    float shift = 0.0f;
+    float recall = 0.0f;
+
+    std::shared_ptr<hip::Context> context;
+    skm_ctx* ctx = nullptr;
+    std::unique_ptr<pruner_t> pruner;
+
+    // Device state (names follow the reference's members, superkmeans.h:1470-1480)
+    dbuf<float> centroids;                     // PDX layout
+    dbuf<float> horizontal_centroids;          // row-major: raw init rows -> sums -> means
+    dbuf<float> prev_centroids;                // centroids the current iteration searches against
+    dbuf<float> partial_horizontal_centroids;  // first vertical_d columns, dense
+    dbuf<float> distances;
+    dbuf<uint32_t> d_cluster_sizes;
+    dbuf<uint32_t> d_assignments;
+    dbuf<float> data_norms;
+    dbuf<float> centroid_norms;
+    dbuf<float> training_data;  // rotated samples (unused when the caller's device buffer is used in place)
+
+    // Host state
+    std::unique_ptr<uint32_t[]> cluster_sizes;
+    std::unique_ptr<size_t[]> sampled_indices;
+    std::vector<float> host_distances;
+
+  public:
+    std::unique_ptr<uint32_t[]> assignments;
+    std::vector<SuperKMeansIterationStats> iteration_stats;
+};
+
+} // namespace skmeans

@@ -180,73 +180,9 @@ static inline float Horizontal(const float* v1, const float* v2, size_t num_dime
 // (adsampling.h:76-85).  Eigen is unavailable, so the factorisation is a textbook Householder QR in
 // double precision; the value sequence of the draws (std::mt19937 + std::normal_distribution<float>,
 // row by row) is the reference's.
-#pragma GCC push_options
-#pragma GCC optimize("fp-contract=off")
-static void HouseholderQ(std::vector<double>& a, size_t d, std::vector<float>& q_out) {
-    // a: d x d row-major, overwritten. vs[j] holds the j-th reflector (length d - j), betas[j] its factor.
-    std::vector<std::vector<double>> vs(d);
-    std::vector<double> betas(d, 0.0);
-    std::vector<double> w(d);
-    for (size_t j = 0; j < d; ++j) {
-        const size_t len = d - j;
-        std::vector<double>& v = vs[j];
-        v.resize(len);
-        double norm2 = 0.0;
-        for (size_t r = 0; r < len; ++r) {
-            v[r] = a[(j + r) * d + j];
-            norm2 += v[r] * v[r];
-        }
-        const double norm = std::sqrt(norm2);
-        if (norm == 0.0) {
-            betas[j] = 0.0;
-            continue;
-        }
-        const double alpha = (v[0] >= 0.0) ? -norm : norm;
-        v[0] -= alpha;
-        double vtv = 0.0;
-        for (size_t r = 0; r < len; ++r) vtv += v[r] * v[r];
-        if (vtv == 0.0) {
-            betas[j] = 0.0;
-            continue;
-        }
-        const double beta = 2.0 / vtv;
-        betas[j] = beta;
-        // A[j:, j:] -= beta * v * (v^T A[j:, j:])
-        for (size_t c = j; c < d; ++c) w[c] = 0.0;
-        for (size_t r = 0; r < len; ++r) {
-            const double vr = v[r];
-            const double* row = &a[(j + r) * d];
-            for (size_t c = j; c < d; ++c) w[c] += vr * row[c];
-        }
-        for (size_t r = 0; r < len; ++r) {
-            const double f = beta * v[r];
-            double* row = &a[(j + r) * d];
-            for (size_t c = j; c < d; ++c) row[c] -= f * w[c];
-        }
-    }
-    // Q = H_0 H_1 ... H_{d-1} * I
-    std::vector<double> q(d * d, 0.0);
-    for (size_t i = 0; i < d; ++i) q[i * d + i] = 1.0;
-    for (size_t jj = d; jj-- > 0;) {
-        if (betas[jj] == 0.0) continue;
-        const std::vector<double>& v = vs[jj];
-        const size_t len = d - jj;
-        for (size_t c = 0; c < d; ++c) w[c] = 0.0;
-        for (size_t r = 0; r < len; ++r) {
-            const double vr = v[r];
-            const double* row = &q[(jj + r) * d];
-            for (size_t c = 0; c < d; ++c) w[c] += vr * row[c];
-        }
-        for (size_t r = 0; r < len; ++r) {
-            const double f = betas[jj] * v[r];
-            double* row = &q[(jj + r) * d];
-            for (size_t c = 0; c < d; ++c) row[c] -= f * w[c];
-        }
-    }
-    q_out.resize(d * d);
-    for (size_t i = 0; i < d * d; ++i) q_out[i] = static_cast<float>(q[i]);
-}
-#pragma GCC pop_options
+// Implemented in rotation_matrix.cpp, which is compiled with -ffp-contract=off so that the draws and
+// the factorisation give the same bits under every compiler.
+void MakeRotationMatrix(uint32_t d, uint32_t seed, std::vector<float>& out);
 
 class ADSamplingPruner {
   public:
@@ -257,13 +193,7 @@ class ADSamplingPruner {
     ADSamplingPruner(uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42)
         : num_dimensions(num_dimensions_), epsilon0(epsilon0_) {
         InitializeRatios();
-        std::mt19937 gen(seed);
-        const size_t d = num_dimensions;
-        std::vector<double> a(d * d);
-        std::normal_distribution<float> dist(0.0f, 1.0f);
-        for (uint32_t i = 0; i < d; ++i)
-            for (uint32_t j = 0; j < d; ++j) a[i * d + j] = dist(gen);
-        HouseholderQ(a, d, matrix);
+        MakeRotationMatrix(num_dimensions, seed, matrix);
     }
 
     // adsampling.h:93-99

@@ -55,7 +55,69 @@ _PROTOTYPES = {
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),
+    # include/skm_kmeans.h
+    "skm_kmeans_default_config": (None, [c_void_p, c_int]),
+    "skm_kmeans_create": (c_int, [c_size_t, c_size_t, c_void_p, c_int, POINTER(c_void_p)]),
+    "skm_kmeans_destroy": (c_int, [c_void_p]),
+    "skm_kmeans_train": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
+    "skm_kmeans_train_device": (c_int, [c_void_p, _F, c_size_t, c_void_p]),
+    "skm_kmeans_assign": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
+    "skm_kmeans_assign_device": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, _F]),
+    "skm_kmeans_assign_training_points": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
+    "skm_kmeans_get_n_clusters": (c_int, [c_void_p, POINTER(c_size_t)]),
+    "skm_kmeans_is_trained": (c_int, [c_void_p, POINTER(c_int)]),
+    "skm_kmeans_n_stats": (c_int, [c_void_p, c_int, POINTER(c_size_t)]),
+    "skm_kmeans_get_stats": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),
+    "skm_kmeans_get_assignments": (c_int, [c_void_p, c_void_p, c_size_t]),
+    "skm_kmeans_context": (c_int, [c_void_p, POINTER(c_void_p)]),
+    "skm_dimension_split": (None, [c_size_t, POINTER(c_size_t), POINTER(c_size_t)]),
+    "skm_pruner_tables": (c_int, [c_size_t, c_float, c_uint32, c_void_p, c_void_p]),
 }
+
+
+class KMeansConfig(ctypes.Structure):
+    """skm_kmeans_config (include/skm_kmeans.h)."""
+
+    _fields_ = [
+        ("iters", c_uint32),
+        ("sampling_fraction", c_float),
+        ("max_points_per_cluster", c_uint32),
+        ("n_threads", c_uint32),
+        ("seed", c_uint32),
+        ("use_blas_only", c_int),
+        ("tol", c_float),
+        ("recall_tol", c_float),
+        ("early_termination", c_int),
+        ("sample_queries", c_int),
+        ("objective_k", c_uint64),
+        ("ann_explore_fraction", c_float),
+        ("min_not_pruned_pct", c_float),
+        ("max_not_pruned_pct", c_float),
+        ("adjustment_factor_for_partial_d", c_float),
+        ("unrotate_centroids", c_int),
+        ("verbose", c_int),
+        ("angular", c_int),
+        ("suppress_warnings", c_int),
+        ("data_already_rotated", c_int),
+        ("iters_mesoclustering", c_uint32),
+        ("iters_fineclustering", c_uint32),
+        ("iters_refinement", c_uint32),
+    ]
+
+
+class KMeansIterationStats(ctypes.Structure):
+    """skm_kmeans_iteration_stats (include/skm_kmeans.h)."""
+
+    _fields_ = [
+        ("iteration", c_uint64),
+        ("objective", c_float),
+        ("shift", c_float),
+        ("split", c_uint64),
+        ("recall", c_float),
+        ("not_pruned_pct", c_float),
+        ("partial_d", c_uint32),
+        ("is_gemm_only", c_int),
+    ]
 
 _lib = None
 
@@ -187,6 +249,117 @@ class Context:
             ms, calls = rest.split("/")
             out[name] = (float(ms), int(calls))
         return out
+
+
+class _BorrowedContext(Context):
+    """A Context view over an skm_ctx owned by someone else (never destroyed here)."""
+
+    def __init__(self, handle):
+        self.lib = load()
+        self.handle = handle
+        self._live = []
+
+    def close(self):
+        for a in list(self._live):
+            a.free()
+        self.handle = None
+
+
+class KMeans:
+    """skm_kmeans: the C-ABI face of skmeans::SuperKMeans / HierarchicalSuperKMeans (HIP backend)."""
+
+    def __init__(self, n_clusters, d, hierarchical=False, **cfg):
+        self.lib = load()
+        self.k, self.d, self.hierarchical = int(n_clusters), int(d), bool(hierarchical)
+        self.config = KMeansConfig()
+        self.lib.skm_kmeans_default_config(ctypes.byref(self.config), 1 if hierarchical else 0)
+        for key, val in cfg.items():
+            if not hasattr(self.config, key):
+                raise AttributeError(key)
+            setattr(self.config, key, val)
+        h = c_void_p()
+        self.handle = None
+        check(self.lib.skm_kmeans_create(self.k, self.d, ctypes.byref(self.config), 1 if hierarchical else 0,
+                                         ctypes.byref(h)))
+        self.handle = h.value
+        c = c_void_p()
+        check(self.lib.skm_kmeans_context(self.handle, ctypes.byref(c)))
+        self.ctx = _BorrowedContext(c.value)
+
+    def close(self):
+        if self.handle:
+            self.ctx.close()
+            check(self.lib.skm_kmeans_destroy(self.handle))
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def train(self, data):
+        data = np.ascontiguousarray(data, dtype=np.float32)
+        out = np.empty((self.k, self.d), dtype=np.float32)
+        check(self.lib.skm_kmeans_train(self.handle, data.ctypes.data, data.shape[0], None, 0, out.ctypes.data))
+        return out
+
+    def train_device(self, d_data, n):
+        out = np.empty((self.k, self.d), dtype=np.float32)
+        ptr = d_data.ptr if isinstance(d_data, DeviceArray) else d_data
+        check(self.lib.skm_kmeans_train_device(self.handle, ptr, n, out.ctypes.data))
+        return out
+
+    def assign(self, vectors, centroids):
+        vectors = np.ascontiguousarray(vectors, dtype=np.float32)
+        centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        out = np.empty(vectors.shape[0], dtype=np.uint32)
+        check(self.lib.skm_kmeans_assign(self.handle, vectors.ctypes.data, centroids.ctypes.data, vectors.shape[0],
+                                         centroids.shape[0], out.ctypes.data))
+        return out
+
+    def assign_device(self, d_vectors, d_centroids, n, k, d_out):
+        check(self.lib.skm_kmeans_assign_device(self.handle, d_vectors.ptr, d_centroids.ptr, n, k, d_out.ptr))
+
+    def assign_training_points(self, vectors, centroids):
+        vectors = np.ascontiguousarray(vectors, dtype=np.float32)
+        centroids = np.ascontiguousarray(centroids, dtype=np.float32)
+        out = np.empty(vectors.shape[0], dtype=np.uint32)
+        check(self.lib.skm_kmeans_assign_training_points(self.handle, vectors.ctypes.data, centroids.ctypes.data,
+                                                         vectors.shape[0], centroids.shape[0], out.ctypes.data))
+        return out
+
+    def stats(self, which=0):
+        n = c_size_t()
+        check(self.lib.skm_kmeans_n_stats(self.handle, which, ctypes.byref(n)))
+        arr = (KMeansIterationStats * n.value)()
+        if n.value:
+            check(self.lib.skm_kmeans_get_stats(self.handle, which, arr, n.value))
+        return list(arr)
+
+    def assignments(self, count):
+        out = np.empty(count, dtype=np.uint32)
+        check(self.lib.skm_kmeans_get_assignments(self.handle, out.ctypes.data, count))
+        return out
+
+    @property
+    def is_trained(self):
+        v = c_int()
+        check(self.lib.skm_kmeans_is_trained(self.handle, ctypes.byref(v)))
+        return bool(v.value)
+
+
+def dimension_split(d):
+    h, v = c_size_t(), c_size_t()
+    load().skm_dimension_split(d, ctypes.byref(h), ctypes.byref(v))
+    return h.value, v.value
+
+
+def pruner_tables(d, epsilon0=1.5, seed=42):
+    m = np.empty((d, d), dtype=np.float32)
+    r = np.empty(d + 1, dtype=np.float32)
+    check(load().skm_pruner_tables(d, epsilon0, seed, m.ctypes.data, r.ctypes.data))
+    return m, r
 
 
 def device_count():
