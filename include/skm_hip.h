@@ -152,6 +152,16 @@ int skm_gather_rows(skm_ctx* ctx, const float* d_x, size_t d, const uint64_t* d_
 int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_t* d_local, size_t m,
                             uint32_t offset, uint32_t* d_out);
 
+/* Benchmark / test utility: seeded Gaussian-mixture rows generated in device memory.  Row i (logical
+ * index row_offset + local row) is  s_j * (center_sigma * g(center_seed, u_i, j) + noise_sigma *
+ * g(point_seed, i, j)),  s_j = (j + 1)^(-decay_exponent),  u_i = hash(i) mod n_centers (n_centers == 0:
+ * pure noise), optionally L2-normalised.  Every value depends only on (seeds, i, j), so any slice can
+ * be regenerated.  The reference's generator for its tests is MakeBlobs (pdx/utils.h:74-123), which
+ * fills host memory from std::mt19937; there is no device counterpart in the reference. */
+int skm_synth_gaussian_mixture(skm_ctx* ctx, float* d_out, size_t n, size_t d, size_t row_offset,
+                               uint32_t n_centers, uint32_t center_seed, uint32_t point_seed,
+                               float center_sigma, float noise_sigma, float decay_exponent, int normalize);
+
 #ifdef __cplusplus
 }
 #endif

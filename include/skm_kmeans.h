@@ -98,6 +98,13 @@ int skm_kmeans_get_assignments(skm_kmeans* km, uint32_t* h_out, size_t count);
 /* The device context of the object: use it for skm_malloc / skm_upload of device-resident inputs
  * and for the per-stage device timers. */
 int skm_kmeans_context(skm_kmeans* km, skm_ctx** out);
+/* Pruning accounting (no counterpart in the reference): when enabled before Train, every pruned
+ * iteration records the number of (point, centroid) pairs entering each pruning step.
+ * skm_kmeans_get_prune_accounting copies row `iteration` (0-based over pruned iterations) into
+ * h_out (capacity entries) and writes the row length to out_len; out_rows receives the row count. */
+int skm_kmeans_set_prune_accounting(skm_kmeans* km, int enabled);
+int skm_kmeans_get_prune_accounting(skm_kmeans* km, size_t iteration, uint64_t* h_out, size_t capacity,
+                                    size_t* out_len, size_t* out_rows);
 /* PDXLayout::GetDimensionSplit (pdx/layout.h:115-140) as used by the host code. */
 void skm_dimension_split(size_t d, size_t* out_horizontal_d, size_t* out_vertical_d);
 /* ADSamplingPruner matrix and ratios as built by the host code for (d, epsilon0, seed): fills

@@ -265,6 +265,16 @@ class SuperKMeans {
     /** Host copy of the per-point squared distances of the last training iteration. */
     [[nodiscard]] distance_t* GetDistancesPointer() { return host_distances.data(); }
     [[nodiscard]] skm_ctx* GetContext() const noexcept { return ctx; }
+    /**
+     * When enabled, every pruned iteration also records how many (point, centroid) pairs entered
+     * each pruning step (first test, each 64-dimension block, the [d', vertical_d) step); one row per
+     * pruned iteration is appended to the returned table.  Used to state the algorithmic bytes of the
+     * pruning stage; off by default because it adds atomics to the kernel.
+     */
+    void SetCollectPruneAccounting(bool on) noexcept { collect_prune_accounting = on; }
+    [[nodiscard]] const std::vector<std::vector<uint64_t>>& GetPruneAccounting() const noexcept {
+        return prune_accounting;
+    }
 
     [[nodiscard]] static ClusterBalanceStats GetClustersBalanceStats(const uint32_t* assignments_in, size_t n_samples_in,
                                                                      size_t n_clusters_in) {
@@ -383,10 +393,14 @@ class SuperKMeans {
                                        centroid_norms.get(), d_assignments.get(), distances.get()));
         } else {
             hip::Check(skm_norms(ctx, prev_centroids.get(), k, d, partial_d, centroid_norms.get()));
+            std::vector<uint64_t> stage_pairs;
+            if (collect_prune_accounting) stage_pairs.assign((d - vertical_d) / H_DIM_SIZE + 2, 0);
             hip::Check(skm_assign_pruned(ctx, data_to_cluster, n_samples_, prev_centroids.get(), centroids.get(),
                                          partial_horizontal_centroids.get(), k, d, vertical_d, partial_d,
                                          pruner->DeviceRatios(), data_norms.get(), centroid_norms.get(),
-                                         d_assignments.get(), distances.get(), &not_pruned_total, nullptr));
+                                         d_assignments.get(), distances.get(), &not_pruned_total,
+                                         collect_prune_accounting ? stage_pairs.data() : nullptr));
+            if (collect_prune_accounting) prune_accounting.push_back(std::move(stage_pairs));
         }
         // Sums and counts (zero-filled by the kernel itself for empty clusters).
         hip::Check(skm_update(ctx, data_to_cluster, n_samples_, d, d_assignments.get(), k, horizontal_centroids.get(),
@@ -711,6 +725,8 @@ class SuperKMeans {
     std::unique_ptr<uint32_t[]> cluster_sizes;
     std::unique_ptr<size_t[]> sampled_indices;
     std::vector<float> host_distances;
+    bool collect_prune_accounting = false;
+    std::vector<std::vector<uint64_t>> prune_accounting;
 
   public:
     std::unique_ptr<uint32_t[]> assignments;

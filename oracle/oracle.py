@@ -261,6 +261,14 @@ def arrange_fine_clusters(n_clusters, n_samples, sizes):
     return out
 
 
+def make_blobs(n_samples, n_features, n_centers, normalize=False, cluster_std=1.0, center_spread=10.0, random_state=42):
+    """MakeBlobs (pdx/utils.h:74-123) with one thread."""
+    out = np.empty((n_samples, n_features), dtype=np.float32)
+    load().oracle_make_blobs(c_size_t(n_samples), c_size_t(n_features), c_size_t(n_centers), c_int(1 if normalize else 0),
+                             c_float(cluster_std), c_float(center_spread), c_uint32(random_state), _fp(out))
+    return out
+
+
 def n_mesoclusters(k):
     return load().oracle_n_mesoclusters(c_size_t(k))
 

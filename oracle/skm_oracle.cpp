@@ -1727,6 +1727,37 @@ float oracle_tune_partial_d(const uint64_t* counts, size_t n, size_t k, uint32_t
     return avg;
 }
 
+// MakeBlobs of the reference's test utilities (pdx/utils.h:74-123) as it behaves with one OpenMP
+// thread (its golden data was generated that way, tests/generate_wcss_ground_truth.cpp:26): centres
+// from mt19937(seed) + normal(0, center_spread); points from a second mt19937(seed + 0) that draws,
+// per row, the centre index with uniform_int_distribution<size_t> and then one normal(0, cluster_std)
+// per feature.
+void oracle_make_blobs(size_t n_samples, size_t n_features, size_t n_centers, int normalize, float cluster_std,
+                       float center_spread, uint32_t random_state, float* out) {
+    std::mt19937 gen(random_state);
+    std::normal_distribution<float> center_dist(0.0f, center_spread);
+    std::vector<float> centers(n_centers * n_features);
+    for (size_t i = 0; i < n_centers * n_features; ++i) centers[i] = center_dist(gen);
+    std::uniform_int_distribution<size_t> cluster_dist(0, n_centers - 1);
+    std::normal_distribution<float> point_dist(0.0f, cluster_std);
+    std::mt19937 thread_gen(random_state + 0u);
+    for (size_t i = 0; i < n_samples; ++i) {
+        size_t center_idx = cluster_dist(thread_gen) * n_features;
+        float* row = &out[i * n_features];
+        const float* center = &centers[center_idx];
+        for (size_t j = 0; j < n_features; ++j) row[j] = center[j] + point_dist(thread_gen);
+    }
+    if (normalize) {
+        for (size_t i = 0; i < n_samples; ++i) {
+            float* row = &out[i * n_features];
+            float norm_sq = 0.0f;
+            for (size_t j = 0; j < n_features; ++j) norm_sq += row[j] * row[j];
+            float inv_norm = 1.0f / std::sqrt(norm_sq);
+            for (size_t j = 0; j < n_features; ++j) row[j] *= inv_norm;
+        }
+    }
+}
+
 void oracle_arrange_fine_clusters(size_t n_clusters, size_t n_meso, size_t n_samples, const uint32_t* sizes,
                                   uint64_t* out) {
     std::vector<uint32_t> s(sizes, sizes + n_meso);

@@ -55,6 +55,10 @@ _PROTOTYPES = {
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),
+    "skm_synth_gaussian_mixture": (
+        c_int,
+        [c_void_p, _F, c_size_t, c_size_t, c_size_t, c_uint32, c_uint32, c_uint32, c_float, c_float, c_float, c_int],
+    ),
     # include/skm_kmeans.h
     "skm_kmeans_default_config": (None, [c_void_p, c_int]),
     "skm_kmeans_create": (c_int, [c_size_t, c_size_t, c_void_p, c_int, POINTER(c_void_p)]),
@@ -70,6 +74,9 @@ _PROTOTYPES = {
     "skm_kmeans_get_stats": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),
     "skm_kmeans_get_assignments": (c_int, [c_void_p, c_void_p, c_size_t]),
     "skm_kmeans_context": (c_int, [c_void_p, POINTER(c_void_p)]),
+    "skm_kmeans_set_prune_accounting": (c_int, [c_void_p, c_int]),
+    "skm_kmeans_get_prune_accounting": (
+        c_int, [c_void_p, c_size_t, c_void_p, c_size_t, POINTER(c_size_t), POINTER(c_size_t)]),
     "skm_dimension_split": (None, [c_size_t, POINTER(c_size_t), POINTER(c_size_t)]),
     "skm_pruner_tables": (c_int, [c_size_t, c_float, c_uint32, c_void_p, c_void_p]),
 }
@@ -336,6 +343,21 @@ class KMeans:
         if n.value:
             check(self.lib.skm_kmeans_get_stats(self.handle, which, arr, n.value))
         return list(arr)
+
+    def set_prune_accounting(self, on=True):
+        check(self.lib.skm_kmeans_set_prune_accounting(self.handle, 1 if on else 0))
+
+    def prune_accounting(self):
+        """List (one entry per pruned iteration) of arrays of pairs entering each pruning step."""
+        rows, ln = c_size_t(), c_size_t()
+        check(self.lib.skm_kmeans_get_prune_accounting(self.handle, 0, None, 0, ctypes.byref(ln), ctypes.byref(rows)))
+        out = []
+        for it in range(rows.value):
+            buf = np.zeros(max(ln.value, 1), dtype=np.uint64)
+            check(self.lib.skm_kmeans_get_prune_accounting(self.handle, it, buf.ctypes.data, buf.size,
+                                                           ctypes.byref(ln), ctypes.byref(rows)))
+            out.append(buf[: ln.value].copy())
+        return out
 
     def assignments(self, count):
         out = np.empty(count, dtype=np.uint32)

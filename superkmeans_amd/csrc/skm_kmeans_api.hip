@@ -234,6 +234,26 @@ int skm_kmeans_context(skm_kmeans* km, skm_ctx** out) {
     return SKM_OK;
 }
 
+int skm_kmeans_set_prune_accounting(skm_kmeans* km, int enabled) {
+    if (!km) return skm::set_error(SKM_ERR_INVALID, "null argument");
+    km->base()->SetCollectPruneAccounting(enabled != 0);
+    return SKM_OK;
+}
+
+int skm_kmeans_get_prune_accounting(skm_kmeans* km, size_t iteration, uint64_t* h_out, size_t capacity,
+                                    size_t* out_len, size_t* out_rows) {
+    if (!km) return skm::set_error(SKM_ERR_INVALID, "null argument");
+    const auto& table = km->base()->GetPruneAccounting();
+    if (out_rows) *out_rows = table.size();
+    if (out_len) *out_len = 0;
+    if (iteration >= table.size()) return SKM_OK;
+    const auto& row = table[iteration];
+    if (out_len) *out_len = row.size();
+    if (h_out)
+        for (size_t i = 0; i < row.size() && i < capacity; ++i) h_out[i] = row[i];
+    return SKM_OK;
+}
+
 void skm_dimension_split(size_t d, size_t* out_horizontal_d, size_t* out_vertical_d) {
     const auto s = skmeans::PDXLayout<>::GetDimensionSplit(d);
     if (out_horizontal_d) *out_horizontal_d = s.horizontal_d;
