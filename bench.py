@@ -42,6 +42,9 @@ def main():
     ap.add_argument("--cpu-train-points", type=int, default=65536)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-train", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain row-copy kernel of known size (1 GiB read + 1 GiB write) three times; "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE hardware counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every box of this build has a single MI355X and the hot path "
@@ -49,6 +52,20 @@ def main():
         sys.exit(2)
 
     from superkmeans_amd import _capi
+
+    if args.copy_calibration:
+        ctx = _capi.Context(0)
+        rows, width = 1 << 18, 1024
+        src, dst = ctx.empty((rows, width)), ctx.empty((rows, width))
+        index = ctx.array(np.arange(rows, dtype=np.uint64))
+        _capi.check(ctx.lib.skm_fill_u32(ctx.handle, src.ptr, 0x3f800000, rows * width))
+        for _ in range(3):
+            _capi.check(ctx.lib.skm_gather_rows(ctx.handle, src.ptr, width, index.ptr, rows, dst.ptr, None, None))
+        ctx.sync()
+        print(json.dumps({"copy_calibration": "gather_rows_kernel", "bytes_read": rows * width * 4 + rows * 8,
+                          "bytes_written": rows * width * 4, "launches": 3}))
+        ctx.close()
+        return
 
     n, d, k = args.n, args.d, args.k
     cfg = dict(iters=args.train_iters, sampling_fraction=1.0, early_termination=0, seed=42, suppress_warnings=1)
