@@ -70,10 +70,14 @@ __device__ __forceinline__ void tile_of_block(const GemmOperands& g, int bid, in
     tm = band * 8 + in_band % rows_in_band;
 }
 
-template <bool VEC>
+// Four consecutive operand columns starting at k.  GUARD: columns at or past K read as zero (last,
+// partial BK step, and every step of the scalar path).
+template <bool VEC, bool GUARD>
 __device__ __forceinline__ floatx4 load_k4(const float* row, int k, int K) {
     floatx4 v;
-    if (VEC) {
+    if (VEC && !GUARD) {
+        v = *reinterpret_cast<const floatx4*>(row + k);
+    } else if (VEC) {
         if (k + 3 < K) {
             v = *reinterpret_cast<const floatx4*>(row + k);
         } else {
@@ -91,8 +95,9 @@ __device__ __forceinline__ floatx4 load_k4(const float* row, int k, int K) {
     return v;
 }
 
-// Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are
-// 16-byte aligned so operand slices can be fetched with dwordx4 loads.
+// Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are 16-byte aligned so operand
+// slices can be fetched with dwordx4 loads; then every full BK step is fetched without any guard (the
+// eight loads of a thread are issued back to back) and only a trailing partial step is guarded.
 template <bool VEC>
 __device__ __forceinline__ void gemm_tile(
     const GemmOperands& g, int tm, int tn, float* lds, WaveAcc& acc
@@ -115,8 +120,8 @@ __device__ __forceinline__ void gemm_tile(
         int rb = tn * GEMM_TN + ld_row + 32 * p;
         ra = ra < g.M ? ra : g.M - 1;  // clamp: duplicates are masked by the epilogue
         rb = rb < g.N ? rb : g.N - 1;
-        a_rows[p] = g.A + (int64_t) ra * g.lda;
-        b_rows[p] = g.B + (int64_t) rb * g.ldb;
+        a_rows[p] = g.A + (int64_t) ra * g.lda + ld_k;
+        b_rows[p] = g.B + (int64_t) rb * g.ldb + ld_k;
     }
     floatx4 ra[4], rb[4];
 
@@ -128,16 +133,26 @@ __device__ __forceinline__ void gemm_tile(
             for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
 
     const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;
+    const int nk_full = VEC ? g.K / GEMM_BK : 0;  // steps that need no guard
 
+    if (nk_full > 0) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        ra[p] = load_k4<VEC>(a_rows[p], ld_k, g.K);
-        rb[p] = load_k4<VEC>(b_rows[p], ld_k, g.K);
+        for (int p = 0; p < 4; ++p) {
+            ra[p] = load_k4<VEC, false>(a_rows[p], 0, g.K);
+            rb[p] = load_k4<VEC, false>(b_rows[p], 0, g.K);
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, ld_k, g.K);
+            rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, ld_k, g.K);
+        }
     }
+    const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-        *reinterpret_cast<floatx4*>(&As[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = ra[p];
-        *reinterpret_cast<floatx4*>(&Bs[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = rb[p];
+        *reinterpret_cast<floatx4*>(&As[st_off + 32 * p * GEMM_LDS_STRIDE]) = ra[p];
+        *reinterpret_cast<floatx4*>(&Bs[st_off + 32 * p * GEMM_LDS_STRIDE]) = rb[p];
     }
     __syncthreads();
 
@@ -146,21 +161,37 @@ __device__ __forceinline__ void gemm_tile(
         const int cur = kt & 1;
         const bool more = (kt + 1) < nk;
         if (more) {
-            const int k0 = (kt + 1) * GEMM_BK + ld_k;
+            const int k0 = (kt + 1) * GEMM_BK;
+            if (kt + 1 < nk_full) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                ra[p] = load_k4<VEC>(a_rows[p], k0, g.K);
-                rb[p] = load_k4<VEC>(b_rows[p], k0, g.K);
+                for (int p = 0; p < 4; ++p) {
+                    ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+                    rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
+                    rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
+                }
             }
         }
         const float* as = As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off;
         const float* bs = Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off;
+        floatx4 a0 = *reinterpret_cast<const floatx4*>(as);
+        floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
+        floatx4 b0 = *reinterpret_cast<const floatx4*>(bs);
+        floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
 #pragma unroll
         for (int kg = 0; kg < GEMM_BK / 8; ++kg) {
-            floatx4 a0 = *reinterpret_cast<const floatx4*>(as + kg * 8);
-            floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + kg * 8);
-            floatx4 b0 = *reinterpret_cast<const floatx4*>(bs + kg * 8);
-            floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + kg * 8);
+            // Fragments of the next group of 8 columns are requested before this group's MFMAs.
+            floatx4 na0, na1, nb0, nb1;
+            if (kg + 1 < GEMM_BK / 8) {
+                na0 = *reinterpret_cast<const floatx4*>(as + (kg + 1) * 8);
+                na1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
+                nb0 = *reinterpret_cast<const floatx4*>(bs + (kg + 1) * 8);
+                nb1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
@@ -168,14 +199,17 @@ __device__ __forceinline__ void gemm_tile(
                 acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
                 acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
             }
+            if (kg + 1 < GEMM_BK / 8) {
+                a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+            }
         }
         if (more) {
-            float* asn = As + (cur ^ 1) * GEMM_TM * GEMM_LDS_STRIDE;
-            float* bsn = Bs + (cur ^ 1) * GEMM_TN * GEMM_LDS_STRIDE;
+            float* asn = As + (cur ^ 1) * GEMM_TM * GEMM_LDS_STRIDE + st_off;
+            float* bsn = Bs + (cur ^ 1) * GEMM_TN * GEMM_LDS_STRIDE + st_off;
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                *reinterpret_cast<floatx4*>(&asn[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = ra[p];
-                *reinterpret_cast<floatx4*>(&bsn[(ld_row + 32 * p) * GEMM_LDS_STRIDE + ld_k]) = rb[p];
+                *reinterpret_cast<floatx4*>(&asn[32 * p * GEMM_LDS_STRIDE]) = ra[p];
+                *reinterpret_cast<floatx4*>(&bsn[32 * p * GEMM_LDS_STRIDE]) = rb[p];
             }
         }
         __syncthreads();
