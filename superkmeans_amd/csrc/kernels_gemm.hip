@@ -182,6 +182,92 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
 }
 
 // ---------------------------------------------------------------------------------------------
+// Partial distances with the first pruning test fused into the epilogue.  Same operand roles as the
+// argmin kernel (one point per lane).  A (point, centroid) pair is emitted only when its partial
+// distance is below thr0[point] = seed distance * ratios[d'], the loosest threshold that point can
+// ever see (its best distance only shrinks from batch to batch, batch_computers.h:372-380), so the
+// emitted set is a superset of the reference's survivors of every batch; the pruning kernel re-applies
+// the exact per-batch threshold.  Pairs go to a per-point list of `cap` slots; the per-point counter
+// keeps counting past `cap` so that overflowing points can be detected and redone densely.
+// ---------------------------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
+    GemmOperands g, const float* __restrict__ xnorm, const float* __restrict__ cnorm,
+    const float* __restrict__ thr0, uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap
+) {
+    extern __shared__ float lds[];
+    int tm, tn;
+    tile_of_block(g, blockIdx.x, tm, tn);
+    WaveAcc acc;
+    gemm_tile<VEC>(g, tm, tn, lds, acc);
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int m0 = tm * GEMM_TM + (wave >> 1) * 64;
+    const int n0 = tn * GEMM_TN + (wave & 1) * 64;
+    if (m0 >= g.M) return;
+    float cn[2][16];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = m0 + acc_row(mb, r, lane);
+            cn[mb][r] = (m < g.M) ? cnorm[m] : 0.0f;
+        }
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        const int n = n0 + acc_col(nb, lane);
+        if (n >= g.N) continue;
+        const float xn = xnorm[n];
+        const float thr = thr0[n];
+        uint32_t pass = 0;  // bit (mb * 16 + r)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + acc_row(mb, r, lane);
+                const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn) + cn[mb][r];
+                acc.v[mb][nb][r] = v;
+                if (m < g.M && v < thr) pass |= 1u << (mb * 16 + r);
+            }
+        if (pass) {
+            const uint32_t cnt = (uint32_t) __popc(pass);
+            uint32_t slot = atomicAdd(&cand_count[n], cnt);
+            uint2* list = cand + (int64_t) n * cap;
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    if (pass & (1u << (mb * 16 + r))) {
+                        if (slot < cap)
+                            list[slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
+                        ++slot;
+                    }
+                }
+        }
+    }
+}
+
+int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
+                           const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
+                           uint2* cand, uint32_t cap) {
+    if (k <= 0 || n <= 0 || partial_d <= 0) return SKM_OK;
+    GemmOperands g;
+    g.A = C; g.B = X; g.M = k; g.N = n; g.K = partial_d; g.lda = ld; g.ldb = ld;
+    g.tiles_m = (k + GEMM_TM - 1) / GEMM_TM;
+    g.tiles_n = (n + GEMM_TN - 1) / GEMM_TN;
+    const long long total = (long long) g.tiles_m * g.tiles_n;
+    if (total > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
+    const size_t lds_bytes = GEMM_LDS_FLOATS * sizeof(float);
+    dim3 grid((unsigned) total), block(GEMM_THREADS);
+    if (gemm_operands_vectorizable(g))
+        SKM_LAUNCH_GEMM((gemm_candidates_kernel<true>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
+    else
+        SKM_LAUNCH_GEMM((gemm_candidates_kernel<false>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
+    return check_hip(hipGetLastError(), "gemm_candidates_kernel launch");
+}
+
+// ---------------------------------------------------------------------------------------------
 // Sequential merge of granule minima, reproducing batch_computers.h:118,162-167:
 //   out = FLT_MAX; for each batch of 1024 centroids in order:
 //       m = first minimum of the batch;  if (m < out) { out = max(0, m); idx = argmin; }

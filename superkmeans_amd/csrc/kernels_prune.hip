@@ -236,6 +236,298 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Seed of the pruned search: squared distance of every point to its previous assignment over all d
+// dimensions (batch_computers.h:372-377) and the loosest first-test threshold derived from it.
+// ---------------------------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
+    const float* __restrict__ x, const float* __restrict__ c, const uint32_t* __restrict__ idx, int n, int d,
+    const float* __restrict__ ratios, int partial_d, float* __restrict__ best0, float* __restrict__ thr0
+) {
+    const int lane = threadIdx.x & 63;
+    const int p = blockIdx.x * PRUNE_WAVES + (threadIdx.x >> 6);
+    if (p >= n) return;
+    const float* xq = x + (int64_t) p * d;
+    const float* cp = c + (int64_t) idx[p] * d;
+    float s = 0.0f;
+    if (VEC) {
+        for (int t = lane * 4; t < d; t += 256) {
+            const float4 xv = *reinterpret_cast<const float4*>(xq + t);
+            const float4 cv = *reinterpret_cast<const float4*>(cp + t);
+            float e;
+            e = cv.x - xv.x; s += e * e;
+            e = cv.y - xv.y; s += e * e;
+            e = cv.z - xv.z; s += e * e;
+            e = cv.w - xv.w; s += e * e;
+        }
+    } else {
+        for (int t = lane; t < d; t += 64) {
+            const float e = cp[t] - xq[t];
+            s += e * e;
+        }
+    }
+    s = wave_sum(s);
+    if (lane == 0) {
+        best0[p] = s;
+        thr0[p] = s * ratios[partial_d];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Pruned search over per-point candidate lists (see gemm_candidates_kernel).  Identical to
+// prune_kernel except for the first test of a batch, which filters the point's candidates that
+// belong to the batch with the exact threshold best * ratios[d'] instead of scanning 1024 dense
+// partial distances.  Candidates arrive in no particular order; every later step is order
+// independent (thresholds are fixed inside a batch, the final minimum breaks ties by position).
+// Batches that hold no candidate are skipped: they would prune everything (count 0) anyway.
+// Points whose list overflowed (count > cap) are left untouched for the dense path.
+// ---------------------------------------------------------------------------------------------
+struct PruneListArgs {
+    const uint2* cand;            // n_chunk x cap {centroid index, partial distance bits}
+    const uint32_t* cand_count;   // n_chunk
+    uint32_t cap;
+    const float* best0;           // seed distances
+    const float* x;
+    const float* pdx;
+    const float* aux;
+    const float* ratios;
+    uint32_t* idx;
+    float* dist;
+    uint32_t* not_pruned;
+    unsigned long long* stage_pairs;
+    int n, k, d, vertical_d, partial_d;
+};
+
+template <bool VEC>
+__global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListArgs a) {
+    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
+    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int p = blockIdx.x * PRUNE_WAVES + wave;
+    if (p >= a.n) return;
+    const uint32_t n_cand = a.cand_count[p];
+    if (n_cand > a.cap) return;  // handled densely by the caller
+    uint16_t* pos = s_pos[wave];
+    float* acc = s_acc[wave];
+    const int d = a.d, V = a.vertical_d, dp = a.partial_d;
+    const int n_hblocks = (d - V) / SKM_H_DIM_SIZE;
+    const float* xq = a.x + (int64_t) p * d;
+    const uint2* list = a.cand + (int64_t) p * a.cap;
+    const int sub = lane & 15, grp = lane >> 4;
+
+    uint32_t best_idx = a.idx[p];
+    float best = a.best0[p];
+    uint32_t not_pruned_total = 0;
+
+    // Smallest batch that holds a candidate.
+    uint32_t jb = 0xffffffffu;
+    for (uint32_t s0 = 0; s0 < n_cand; s0 += 64) {
+        const uint32_t s = s0 + lane;
+        if (s < n_cand) {
+            const uint32_t b = list[s].x / SKM_Y_BATCH_SIZE;
+            jb = b < jb ? b : jb;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t) __shfl_xor((int) jb, off);
+        jb = o < jb ? o : jb;
+    }
+
+    while (jb != 0xffffffffu) {
+        const int base = (int) jb * SKM_Y_BATCH_SIZE;
+        const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
+        const uint32_t prev_top_1 = best_idx;
+        float thr = best * a.ratios[dp];
+        int cnt = 0;
+        uint32_t next_jb = 0xffffffffu;
+        for (uint32_t s0 = 0; s0 < n_cand; s0 += 64) {
+            const uint32_t s = s0 + lane;
+            bool keep = false;
+            uint2 e = make_uint2(0u, 0u);
+            if (s < n_cand) {
+                e = list[s];
+                const uint32_t b = e.x / SKM_Y_BATCH_SIZE;
+                if (b == jb) {
+                    keep = __uint_as_float(e.y) < thr;
+                } else if (b > jb && b < next_jb) {
+                    next_jb = b;
+                }
+            }
+            const unsigned long long mask = __ballot(keep);
+            if (keep) {
+                const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+                pos[slot] = (uint16_t) (e.x - (uint32_t) base);
+                acc[slot] = __uint_as_float(e.y);
+            }
+            cnt += __popcll(mask);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t o = (uint32_t) __shfl_xor((int) next_jb, off);
+            next_jb = o < next_jb ? o : next_jb;
+        }
+        jb = next_jb;
+        not_pruned_total += (uint32_t) cnt;
+        if (a.stage_pairs && lane == 0 && cnt) atomicAdd(&a.stage_pairs[0], (unsigned long long) cnt);
+        if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
+        if (cnt == 0) continue;
+
+        const float* chunk = a.pdx + (int64_t) base * d;
+        int dims_seen = dp;
+        for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
+            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + hb], (unsigned long long) cnt);
+            const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
+            const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
+            float4 xv;
+            if (VEC) {
+                xv = *reinterpret_cast<const float4*>(xb + sub * 4);
+            } else {
+                xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
+            }
+            for (int s0 = 0; s0 < cnt; s0 += 4) {
+                const int s = s0 + grp;
+                const bool in = s < cnt;
+                const int cpos = in ? pos[s] : pos[0];
+                const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                float4 cv;
+                if (VEC) {
+                    cv = *reinterpret_cast<const float4*>(cb);
+                } else {
+                    cv = make_float4(cb[0], cb[1], cb[2], cb[3]);
+                }
+                float e, part = 0.0f;
+                e = xv.x - cv.x; part += e * e;
+                e = xv.y - cv.y; part += e * e;
+                e = xv.z - cv.z; part += e * e;
+                e = xv.w - cv.w; part += e * e;
+                part = group16_sum(part);
+                if (in && sub == 0) acc[s] += part;
+            }
+            dims_seen += SKM_H_DIM_SIZE;
+            thr = best * a.ratios[dims_seen];
+            cnt = compact_survivors(pos, acc, cnt, thr, lane);
+        }
+        if (cnt > 0 && dp < V) {
+            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + n_hblocks], (unsigned long long) cnt);
+            const int left = V - dp;
+            for (int s0 = 0; s0 < cnt; s0 += 4) {
+                const int s = s0 + grp;
+                const bool in = s < cnt;
+                const int cpos = in ? pos[s] : pos[0];
+                const float* cb = a.aux + (int64_t) (base + cpos) * V + dp;
+                float part = 0.0f;
+                for (int t = sub; t < left; t += 16) {
+                    const float e = xq[dp + t] - cb[t];
+                    part += e * e;
+                }
+                part = group16_sum(part);
+                if (in && sub == 0) acc[s] += part;
+            }
+            thr = best * a.ratios[d];
+            cnt = compact_survivors(pos, acc, cnt, thr, lane);
+        }
+        if (cnt > 0) {
+            float bv = FLT_MAX;
+            int bp = 0x7fffffff;
+            for (int s = lane; s < cnt; s += 64) {
+                const float v = acc[s];
+                const int q = pos[s];
+                if (v < bv || (v == bv && q < bp)) {
+                    bv = v;
+                    bp = q;
+                }
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(bv, off);
+                const int op = __shfl_xor(bp, off);
+                if (ov < bv || (ov == bv && op < bp)) {
+                    bv = ov;
+                    bp = op;
+                }
+            }
+            if (bp != 0x7fffffff && bv < best) {
+                best = bv;
+                best_idx = (uint32_t) (base + bp);
+            }
+        }
+    }
+    if (lane == 0) {
+        a.idx[p] = best_idx;
+        a.dist[p] = best;
+        a.not_pruned[p] = not_pruned_total;
+    }
+}
+
+// Ids (chunk-local) of the points whose candidate list overflowed.
+__global__ __launch_bounds__(256) void collect_overflow_kernel(
+    const uint32_t* __restrict__ cand_count, int n, uint32_t cap, uint64_t* __restrict__ ids, uint32_t* __restrict__ n_over
+) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && cand_count[i] > cap) ids[atomicAdd(n_over, 1u)] = (uint64_t) i;
+}
+
+__global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ in, const uint64_t* __restrict__ ids, int m, uint32_t* __restrict__ out) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < m) out[j] = in[ids[j]];
+}
+
+__global__ __launch_bounds__(256) void scatter_u32_kernel(const uint32_t* __restrict__ in, const uint64_t* __restrict__ ids, int m, uint32_t* __restrict__ out) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j < m) out[ids[j]] = in[j];
+}
+
+int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
+                         const float* ratios, int partial_d, float* best0, float* thr0) {
+    if (n <= 0) return SKM_OK;
+    const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(c) % 16 == 0);
+    dim3 grid((n + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    if (vec)
+        hipLaunchKernelGGL(seed_distance_kernel<true>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0);
+    else
+        hipLaunchKernelGGL(seed_distance_kernel<false>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0);
+    return check_hip(hipGetLastError(), "seed_distance_kernel launch");
+}
+
+int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
+                      const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
+                      int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
+                      unsigned long long* d_stage_pairs) {
+    if (n_chunk <= 0) return SKM_OK;
+    PruneListArgs a;
+    a.cand = cand; a.cand_count = cand_count; a.cap = cap; a.best0 = best0; a.x = x; a.pdx = pdx; a.aux = aux;
+    a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
+    a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
+    const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
+    dim3 grid((n_chunk + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    if (vec)
+        hipLaunchKernelGGL(prune_list_kernel<true>, grid, block, 0, ctx->stream, a);
+    else
+        hipLaunchKernelGGL(prune_list_kernel<false>, grid, block, 0, ctx->stream, a);
+    return check_hip(hipGetLastError(), "prune_list_kernel launch");
+}
+
+int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t* ids, uint32_t* n_over) {
+    if (n <= 0) return SKM_OK;
+    hipLaunchKernelGGL(collect_overflow_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, cand_count, n, cap, ids, n_over);
+    return check_hip(hipGetLastError(), "collect_overflow_kernel launch");
+}
+
+int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out) {
+    if (m <= 0) return SKM_OK;
+    hipLaunchKernelGGL(gather_u32_kernel, dim3((m + 255) / 256), dim3(256), 0, ctx->stream, in, ids, m, out);
+    return check_hip(hipGetLastError(), "gather_u32_kernel launch");
+}
+
+int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out) {
+    if (m <= 0) return SKM_OK;
+    hipLaunchKernelGGL(scatter_u32_kernel, dim3((m + 255) / 256), dim3(256), 0, ctx->stream, in, ids, m, out);
+    return check_hip(hipGetLastError(), "scatter_u32_kernel launch");
+}
+
 int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
                  const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
                  int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,

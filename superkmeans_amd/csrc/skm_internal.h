@@ -98,4 +98,17 @@ int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const f
                  int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
                  uint32_t* out_not_pruned, unsigned long long* d_stage_pairs);
 
+int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
+                           const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
+                           uint2* cand, uint32_t cap);
+int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
+                         const float* ratios, int partial_d, float* best0, float* thr0);
+int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
+                      const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
+                      int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
+                      unsigned long long* d_stage_pairs);
+int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t* ids, uint32_t* n_over);
+int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
+int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
+
 } // namespace skm

@@ -1,5 +1,13 @@
 // skm_assign_pruned: partial-distance GEMM on the leading d' dimensions followed by the per-point
 // pruned search (reference distance_computers/batch_computers.h:297-409).
+//
+// Per chunk of points:
+//   1. seed_distance_kernel     full distance to the previous assignment -> best0, thr0 = best0 * ratios[d']
+//   2. gemm_candidates_kernel   MFMA partial distances; the epilogue emits only pairs below thr0 into
+//                               per-point lists (nothing dense is written)
+//   3. prune_list_kernel        exact per-batch thresholds, block-wise pruning, best candidate
+//   4. points whose list overflowed are redone with the dense pair gemm_store_kernel + prune_kernel
+//      (same results, more traffic); with sane seeds there are none.
 #include "skm_internal.h"
 
 #include <algorithm>
@@ -10,6 +18,39 @@ int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_
 }
 
 using namespace skm;
+
+namespace {
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Dense path on a contiguous block of points (also the fallback for overflowed points).
+int dense_block(skm_ctx* ctx, const float* d_x, size_t m, const float* d_c, const float* d_pdx, const float* d_aux,
+                size_t k, size_t d, size_t vertical_d, uint32_t partial_d, const float* d_ratios, const float* d_xnorm_p,
+                const float* d_cnorm_p, uint32_t* d_idx, float* d_dist, uint32_t* d_counts, unsigned long long* d_stage) {
+    const size_t ld = align_up(k, 64);
+    size_t sub = ctx->workspace_limit / (ld * sizeof(float));
+    sub = std::max<size_t>(128, (sub / 128) * 128);
+    sub = std::min<size_t>(sub, size_t(1) << 22);
+    void* ws_partial = nullptr;
+    SKM_TRY(workspace(ctx, 0, std::min(sub, m) * ld * sizeof(float), &ws_partial));
+    for (size_t i0 = 0; i0 < m; i0 += sub) {
+        const size_t mm = std::min(sub, m - i0);
+        {
+            ScopedStage st(ctx, "search/blas");
+            SKM_TRY(launch_gemm_store(ctx, d_x + i0 * d, (int) mm, (int64_t) d, d_c, (int) k, (int64_t) d, (int) partial_d,
+                                      (float*) ws_partial, (int64_t) ld, d_xnorm_p + i0, d_cnorm_p));
+        }
+        {
+            ScopedStage st(ctx, "search/pdx");
+            SKM_TRY(launch_prune(ctx, (const float*) ws_partial, (int64_t) ld, d_x + i0 * d, (int) mm, d_c, d_pdx, d_aux,
+                                 (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_idx + i0, d_dist + i0,
+                                 d_counts + i0, d_stage));
+        }
+    }
+    return SKM_OK;
+}
+
+} // namespace
 
 extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, const float* d_pdx,
                                  const float* d_aux, size_t k, size_t d, size_t vertical_d, uint32_t partial_d,
@@ -31,31 +72,78 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     SKM_REQUIRE(partial_d > 0 && partial_d <= vertical_d, "partial_d must be in (0, vertical_d]");
     ScopedStage outer(ctx, "search");
 
-    const size_t ld = ((k + 63) / 64) * 64;
-    size_t chunk = ctx->workspace_limit / (ld * sizeof(float));
+    // Candidate slots per point: a quarter of the centroids (every centroid when there is one batch).
+    const uint32_t cap = (k <= SKM_Y_BATCH_SIZE) ? (uint32_t) align_up(k, 64)
+                                                 : (uint32_t) std::min<size_t>(8192, std::max<size_t>(1024, align_up(k / 4, 64)));
+    size_t chunk = ctx->workspace_limit / (size_t(cap) * sizeof(uint2));
     chunk = std::max<size_t>(128, (chunk / 128) * 128);
     chunk = std::min<size_t>(chunk, size_t(1) << 22);
-    chunk = std::min(chunk, ((n + 127) / 128) * 128);
-    void* ws_partial = nullptr;
-    SKM_TRY(workspace(ctx, 0, std::min(chunk, n) * ld * sizeof(float), &ws_partial));
+    chunk = std::min(chunk, align_up(n, 128));
+    const size_t cn = std::min(chunk, n);
+
     void* ws_counts = nullptr;
     SKM_TRY(workspace(ctx, 1, n * sizeof(uint32_t) + (n_hblocks + 2) * sizeof(unsigned long long) + 64, &ws_counts));
     unsigned long long* d_stage = (unsigned long long*) ws_counts;
     uint32_t* d_counts = (uint32_t*) (d_stage + n_hblocks + 2);
     if (h_out_stage_pairs) SKM_TRY(skm_fill_u32(ctx, d_stage, 0u, 2 * (n_hblocks + 2)));
+    unsigned long long* stage_arg = h_out_stage_pairs ? d_stage : nullptr;
+
+    // Per-chunk scalars: best0, thr0, candidate counts, overflow ids, overflow counter.
+    void* ws_chunk = nullptr;
+    SKM_TRY(workspace(ctx, 2, cn * (3 * sizeof(uint32_t) + sizeof(uint64_t)) + 256, &ws_chunk));
+    uint64_t* d_over_ids = (uint64_t*) ws_chunk;
+    float* d_best0 = (float*) (d_over_ids + cn);
+    float* d_thr0 = d_best0 + cn;
+    uint32_t* d_cand_count = (uint32_t*) (d_thr0 + cn);
+    uint32_t* d_n_over = d_cand_count + cn;
+    void* h_pin = nullptr;
+    SKM_TRY(pinned(ctx, 64, &h_pin));
 
     for (size_t i0 = 0; i0 < n; i0 += chunk) {
         const size_t m = std::min(chunk, n - i0);
+        void* ws_cand = nullptr;
+        SKM_TRY(workspace(ctx, 0, m * size_t(cap) * sizeof(uint2), &ws_cand));
+        const float* xc = d_x + i0 * d;
         {
-            ScopedStage st(ctx, "search/blas");
-            SKM_TRY(launch_gemm_store(ctx, d_x + i0 * d, (int) m, (int64_t) d, d_c, (int) k, (int64_t) d, (int) partial_d,
-                                      (float*) ws_partial, (int64_t) ld, d_xnorm_p + i0, d_cnorm_p));
+            ScopedStage st(ctx, "search/seed");
+            SKM_TRY(launch_seed_distance(ctx, xc, d_c, d_inout_idx + i0, (int) m, (int) d, d_ratios, (int) partial_d,
+                                         d_best0, d_thr0));
+            SKM_TRY(skm_fill_u32(ctx, d_cand_count, 0u, m));
+            SKM_TRY(skm_fill_u32(ctx, d_n_over, 0u, 1));
         }
         {
+            ScopedStage st(ctx, "search/blas");
+            SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
+                                           d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
+        }
+        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, d_over_ids, d_n_over));
+        SKM_HIP_TRY(hipMemcpyAsync(h_pin, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+        {
             ScopedStage st(ctx, "search/pdx");
-            SKM_TRY(launch_prune(ctx, (const float*) ws_partial, (int64_t) ld, d_x + i0 * d, (int) m, d_c, d_pdx, d_aux,
-                                 (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
-                                 d_out_dist + i0, d_counts + i0, h_out_stage_pairs ? d_stage : nullptr));
+            SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
+                                      (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
+                                      d_out_dist + i0, d_counts + i0, stage_arg));
+        }
+        SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        const uint32_t n_over = *(volatile uint32_t*) h_pin;
+        if (n_over > 0) {
+            // Dense redo of the overflowed points: gather them, run the dense pair, scatter the results back.
+            ScopedStage st(ctx, "search/overflow");
+            const size_t mo = n_over;
+            void* ws_o = nullptr;
+            SKM_TRY(workspace(ctx, 3, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
+            float* xo = (float*) ws_o;
+            float* xnorm_o = xo + mo * d;
+            uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
+            float* dist_o = (float*) (idx_o + align_up(mo, 64));
+            uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
+            SKM_TRY(skm_gather_rows(ctx, xc, d, d_over_ids, mo, xo, d_xnorm_p + i0, xnorm_o));
+            SKM_TRY(launch_gather_u32(ctx, d_inout_idx + i0, d_over_ids, (int) mo, idx_o));
+            SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p,
+                                idx_o, dist_o, cnt_o, stage_arg));
+            SKM_TRY(launch_scatter_u32(ctx, idx_o, d_over_ids, (int) mo, d_inout_idx + i0));
+            SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_over_ids, (int) mo, (uint32_t*) (d_out_dist + i0)));
+            SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_over_ids, (int) mo, d_counts + i0));
         }
     }
     if (h_out_not_pruned) {
