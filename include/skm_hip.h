@@ -51,7 +51,8 @@ int skm_device_count(int* out_count);
 int skm_ctx_create(int device, skm_ctx** out_ctx);
 int skm_ctx_destroy(skm_ctx* ctx);
 int skm_sync(skm_ctx* ctx);
-/* Upper bound, in bytes, of the scratch a single stage call may allocate (default 4 GiB). */
+/* Upper bound, in bytes, of the scratch a single stage call may allocate (default 24 GiB of the
+ * 288 GB of HBM: large enough that the headline shapes run as one launch per stage). */
 int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
 
 /* Device memory and transfers (stand in for the reference's std::unique_ptr<float[]> buffers,

@@ -95,6 +95,52 @@ __device__ __forceinline__ floatx4 load_k4(const float* row, int k, int K) {
     return v;
 }
 
+// One full BK step of a wavefront's 64 x 64 quadrant: 4 groups of 8 columns, 16 MFMAs each; the
+// fragments of the next group are requested before the current group's MFMAs.
+__device__ __forceinline__ void mfma_step_full(const float* as, const float* bs, WaveAcc& acc) {
+    floatx4 a0 = *reinterpret_cast<const floatx4*>(as);
+    floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
+    floatx4 b0 = *reinterpret_cast<const floatx4*>(bs);
+    floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
+#pragma unroll
+    for (int kg = 0; kg < GEMM_BK / 8; ++kg) {
+        floatx4 na0, na1, nb0, nb1;
+        if (kg + 1 < GEMM_BK / 8) {
+            na0 = *reinterpret_cast<const floatx4*>(as + (kg + 1) * 8);
+            na1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
+            nb0 = *reinterpret_cast<const floatx4*>(bs + (kg + 1) * 8);
+            nb1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
+            acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
+            acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
+            acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
+        }
+        if (kg + 1 < GEMM_BK / 8) {
+            a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+        }
+    }
+}
+
+// Trailing partial step: only the `kg_live` groups of 8 columns that hold data (the rest is zero).
+__device__ __forceinline__ void mfma_step_tail(const float* as, const float* bs, WaveAcc& acc, int kg_live) {
+    for (int kg = 0; kg < kg_live; ++kg) {
+        const floatx4 a0 = *reinterpret_cast<const floatx4*>(as + kg * 8);
+        const floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + kg * 8);
+        const floatx4 b0 = *reinterpret_cast<const floatx4*>(bs + kg * 8);
+        const floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + kg * 8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
+            acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
+            acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
+            acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
+        }
+    }
+}
+
 // Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are 16-byte aligned so operand
 // slices can be fetched with dwordx4 loads; then every full BK step is fetched without any guard (the
 // eight loads of a thread are issued back to back) and only a trailing partial step is guarded.
@@ -157,7 +203,8 @@ __device__ __forceinline__ void gemm_tile(
     __syncthreads();
 
     const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
-    for (int kt = 0; kt < nk; ++kt) {
+    const int n_full_steps = g.K / GEMM_BK;  // steps whose 32 columns all hold data
+    for (int kt = 0; kt < n_full_steps; ++kt) {
         const int cur = kt & 1;
         const bool more = (kt + 1) < nk;
         if (more) {
@@ -176,33 +223,8 @@ __device__ __forceinline__ void gemm_tile(
                 }
             }
         }
-        const float* as = As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off;
-        const float* bs = Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off;
-        floatx4 a0 = *reinterpret_cast<const floatx4*>(as);
-        floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
-        floatx4 b0 = *reinterpret_cast<const floatx4*>(bs);
-        floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
-#pragma unroll
-        for (int kg = 0; kg < GEMM_BK / 8; ++kg) {
-            // Fragments of the next group of 8 columns are requested before this group's MFMAs.
-            floatx4 na0, na1, nb0, nb1;
-            if (kg + 1 < GEMM_BK / 8) {
-                na0 = *reinterpret_cast<const floatx4*>(as + (kg + 1) * 8);
-                na1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
-                nb0 = *reinterpret_cast<const floatx4*>(bs + (kg + 1) * 8);
-                nb1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
-                acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
-                acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
-                acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
-            }
-            if (kg + 1 < GEMM_BK / 8) {
-                a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
-            }
-        }
+        mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off,
+                       Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off, acc);
         if (more) {
             float* asn = As + (cur ^ 1) * GEMM_TM * GEMM_LDS_STRIDE + st_off;
             float* bsn = Bs + (cur ^ 1) * GEMM_TN * GEMM_LDS_STRIDE + st_off;
@@ -212,6 +234,13 @@ __device__ __forceinline__ void gemm_tile(
                 *reinterpret_cast<floatx4*>(&bsn[32 * p * GEMM_LDS_STRIDE]) = rb[p];
             }
         }
+        __syncthreads();
+    }
+    if (n_full_steps < nk) {
+        const int cur = n_full_steps & 1;
+        mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off,
+                       Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off, acc,
+                       (g.K - n_full_steps * GEMM_BK + 7) / 8);
         __syncthreads();
     }
 }

@@ -190,62 +190,171 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
 // the exact per-batch threshold.  Pairs go to a per-point list of `cap` slots; the per-point counter
 // keeps counting past `cap` so that overflowing points can be detected and redone densely.
 // ---------------------------------------------------------------------------------------------
+// One workgroup owns a tile of 128 points and sweeps every 128-centroid tile in ascending order, so
+//   * a point's candidates are appended batch after batch (a batch of 1024 centroids = 8 consecutive
+//     tiles), which lets the pruning kernel walk its list once;
+//   * ||x||^2 and the thresholds of the workgroup's points stay in registers for the whole sweep, the
+//     128 centroid norms of a tile are staged through LDS: the epilogue issues no global load;
+//   * the first operand slice of tile t+1 is requested during the last MFMA step of tile t and lands
+//     while the epilogue of tile t runs, so neither the prologue nor the epilogue latency is exposed.
+// Workgroups of one XCD sweep the centroid tiles roughly in step and share them through that XCD's L2.
 template <bool VEC>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     GemmOperands g, const float* __restrict__ xnorm, const float* __restrict__ cnorm,
     const float* __restrict__ thr0, uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap
 ) {
     extern __shared__ float lds[];
-    int tm, tn;
-    tile_of_block(g, blockIdx.x, tm, tn);
-    WaveAcc acc;
-    gemm_tile<VEC>(g, tm, tn, lds, acc);
+    float* As = lds;
+    float* Bs = lds + 2 * GEMM_TM * GEMM_LDS_STRIDE;
+    float* cn_s = lds + GEMM_LDS_FLOATS;  // [2][GEMM_TM]
+    // The workgroup is the only writer of its points' lists, so the slot counters live in LDS.
+    uint32_t* cnt_s = reinterpret_cast<uint32_t*>(cn_s + 2 * GEMM_TM);  // [GEMM_TN]
+    const int tn = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int ld_row = tid >> 3;
+    const int ld_k = (tid & 7) * 4;
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int m0 = tm * GEMM_TM + (wave >> 1) * 64;
-    const int n0 = tn * GEMM_TN + (wave & 1) * 64;
-    if (m0 >= g.M) return;
-    float cn[2][16];
+    const float* b_rows[4];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + acc_row(mb, r, lane);
-            cn[mb][r] = (m < g.M) ? cnorm[m] : 0.0f;
-        }
+    for (int p = 0; p < 4; ++p) {
+        int rb = tn * GEMM_TN + ld_row + 32 * p;
+        rb = rb < g.N ? rb : g.N - 1;
+        b_rows[p] = g.B + (int64_t) rb * g.ldb;
+    }
+    // The two points of this lane.
+    int pt[2];
+    float xn[2], thr[2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
-        const int n = n0 + acc_col(nb, lane);
-        if (n >= g.N) continue;
-        const float xn = xnorm[n];
-        const float thr = thr0[n];
-        uint32_t pass = 0;  // bit (mb * 16 + r)
+        pt[nb] = tn * GEMM_TN + wn * 64 + acc_col(nb, lane);
+        const bool valid = pt[nb] < g.N;
+        xn[nb] = valid ? xnorm[pt[nb]] : 0.0f;
+        thr[nb] = valid ? thr0[pt[nb]] : -3.0e38f;  // nothing passes for padding columns
+    }
+
+    const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;
+    const int nk_full = VEC ? g.K / GEMM_BK : 0;
+    floatx4 ra[4], rb[4];
+    float cn_next = 0.0f;
+
+    // Requests operand slice `kt` of centroid tile `tm` (and that tile's norms when kt == 0).
+    auto request = [&](int tm, int kt) {
+        const int k0 = kt * GEMM_BK + ld_k;
+        if (kt < nk_full) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                int r = tm * GEMM_TM + ld_row + 32 * p;
+                r = r < g.M ? r : g.M - 1;
+                ra[p] = load_k4<VEC, false>(g.A + (int64_t) r * g.lda, k0, g.K);
+                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                int r = tm * GEMM_TM + ld_row + 32 * p;
+                r = r < g.M ? r : g.M - 1;
+                ra[p] = load_k4<VEC, true>(g.A + (int64_t) r * g.lda, k0, g.K);
+                rb[p] = load_k4<VEC, true>(b_rows[p], k0, g.K);
+            }
+        }
+        if (kt == 0 && tid < GEMM_TM) {
+            const int m = tm * GEMM_TM + tid;
+            cn_next = m < g.M ? cnorm[m] : 0.0f;
+        }
+    };
+    const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
+    auto publish = [&](int buf) {
+        float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + st_off;
+        float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + st_off;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            *reinterpret_cast<floatx4*>(&as[32 * p * GEMM_LDS_STRIDE]) = ra[p];
+            *reinterpret_cast<floatx4*>(&bs[32 * p * GEMM_LDS_STRIDE]) = rb[p];
+        }
+    };
+
+    int cur = 0;
+    request(0, 0);
+    publish(0);
+    if (tid < GEMM_TM) {
+        cn_s[tid] = cn_next;
+        cnt_s[tid] = 0u;
+    }
+    __syncthreads();
+
+    const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
+    for (int tm = 0; tm < g.tiles_m; ++tm) {
+        WaveAcc acc;
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + acc_row(mb, r, lane);
-                const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn) + cn[mb][r];
-                acc.v[mb][nb][r] = v;
-                if (m < g.M && v < thr) pass |= 1u << (mb * 16 + r);
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
+        const bool next_tile = (tm + 1) < g.tiles_m;
+        for (int kt = 0; kt < nk; ++kt) {
+            const bool inner = (kt + 1) < nk;
+            if (inner) {
+                request(tm, kt + 1);
+            } else if (next_tile) {
+                request(tm + 1, 0);
             }
-        if (pass) {
-            const uint32_t cnt = (uint32_t) __popc(pass);
-            uint32_t slot = atomicAdd(&cand_count[n], cnt);
-            uint2* list = cand + (int64_t) n * cap;
+            const float* as = As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off;
+            const float* bs = Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off;
+            const int k_left = g.K - kt * GEMM_BK;
+            if (k_left >= GEMM_BK) {
+                mfma_step_full(as, bs, acc);
+            } else {
+                mfma_step_tail(as, bs, acc, (k_left + 7) / 8);
+            }
+            if (inner) {
+                publish(cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+
+        // ---- epilogue of tile tm: first pruning test, candidates appended to the per-point lists ----
+        const float* cns = cn_s + (tm & 1) * GEMM_TM + wm * 64;
+        const int m0 = tm * GEMM_TM + wm * 64;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            uint32_t pass = 0;  // bit (mb * 16 + r)
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    if (pass & (1u << (mb * 16 + r))) {
-                        if (slot < cap)
-                            list[slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
-                        ++slot;
-                    }
+                    const int ml = acc_row(mb, r, lane);
+                    const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn[nb]) + cns[ml];
+                    acc.v[mb][nb][r] = v;
+                    if (m0 + ml < g.M && v < thr[nb]) pass |= 1u << (mb * 16 + r);
                 }
+            if (pass) {
+                uint32_t slot = atomicAdd(&cnt_s[wn * 64 + acc_col(nb, lane)], (uint32_t) __popc(pass));
+                uint2* list = cand + (int64_t) pt[nb] * cap;
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        if (pass & (1u << (mb * 16 + r))) {
+                            if (slot < cap)
+                                list[slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
+                            ++slot;
+                        }
+                    }
+            }
         }
+        if (next_tile) {
+            publish(cur ^ 1);
+            if (tid < GEMM_TM) cn_s[((tm + 1) & 1) * GEMM_TM + tid] = cn_next;
+        }
+        __syncthreads();
+        cur ^= 1;
     }
+    if (tid < GEMM_TN && tn * GEMM_TN + tid < g.N) cand_count[tn * GEMM_TN + tid] = cnt_s[tid];
 }
 
 int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
@@ -256,10 +365,8 @@ int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, 
     g.A = C; g.B = X; g.M = k; g.N = n; g.K = partial_d; g.lda = ld; g.ldb = ld;
     g.tiles_m = (k + GEMM_TM - 1) / GEMM_TM;
     g.tiles_n = (n + GEMM_TN - 1) / GEMM_TN;
-    const long long total = (long long) g.tiles_m * g.tiles_n;
-    if (total > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
-    const size_t lds_bytes = GEMM_LDS_FLOATS * sizeof(float);
-    dim3 grid((unsigned) total), block(GEMM_THREADS);
+    const size_t lds_bytes = (GEMM_LDS_FLOATS + 2 * GEMM_TM + GEMM_TN) * sizeof(float);
+    dim3 grid((unsigned) g.tiles_n), block(GEMM_THREADS);
     if (gemm_operands_vectorizable(g))
         SKM_LAUNCH_GEMM((gemm_candidates_kernel<true>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
     else

@@ -462,12 +462,13 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
     }
 }
 
-// Ids (chunk-local) of the points whose candidate list overflowed.
+// Appends the ids (id_offset + chunk-local index) of the points whose candidate list overflowed.
 __global__ __launch_bounds__(256) void collect_overflow_kernel(
-    const uint32_t* __restrict__ cand_count, int n, uint32_t cap, uint64_t* __restrict__ ids, uint32_t* __restrict__ n_over
+    const uint32_t* __restrict__ cand_count, int n, uint32_t cap, uint64_t id_offset, uint64_t* __restrict__ ids,
+    uint32_t* __restrict__ n_over
 ) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n && cand_count[i] > cap) ids[atomicAdd(n_over, 1u)] = (uint64_t) i;
+    if (i < n && cand_count[i] > cap) ids[atomicAdd(n_over, 1u)] = id_offset + (uint64_t) i;
 }
 
 __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ in, const uint64_t* __restrict__ ids, int m, uint32_t* __restrict__ out) {
@@ -510,9 +511,11 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     return check_hip(hipGetLastError(), "prune_list_kernel launch");
 }
 
-int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t* ids, uint32_t* n_over) {
+int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
+                            uint64_t* ids, uint32_t* n_over) {
     if (n <= 0) return SKM_OK;
-    hipLaunchKernelGGL(collect_overflow_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, cand_count, n, cap, ids, n_over);
+    hipLaunchKernelGGL(collect_overflow_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, cand_count, n, cap,
+                       id_offset, ids, n_over);
     return check_hip(hipGetLastError(), "collect_overflow_kernel launch");
 }
 

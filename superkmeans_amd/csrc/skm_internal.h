@@ -23,7 +23,7 @@ struct skm_pending_interval {
 struct skm_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
-    size_t workspace_limit = size_t(4) << 30;
+    size_t workspace_limit = size_t(24) << 30;
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
     void* ws[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t ws_bytes[4] = {0, 0, 0, 0};
@@ -107,7 +107,8 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs);
-int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t* ids, uint32_t* n_over);
+int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
+                            uint64_t* ids, uint32_t* n_over);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 

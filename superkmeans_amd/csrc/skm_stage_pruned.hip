@@ -6,8 +6,9 @@
 //   2. gemm_candidates_kernel   MFMA partial distances; the epilogue emits only pairs below thr0 into
 //                               per-point lists (nothing dense is written)
 //   3. prune_list_kernel        exact per-batch thresholds, block-wise pruning, best candidate
-//   4. points whose list overflowed are redone with the dense pair gemm_store_kernel + prune_kernel
-//      (same results, more traffic); with sane seeds there are none.
+// After the last chunk, the points whose list overflowed (loose seeds, points with no centroid nearby)
+// are gathered and redone with the dense pair gemm_store_kernel + prune_kernel: same results, more
+// traffic, and only for those points.
 #include "skm_internal.h"
 
 #include <algorithm>
@@ -36,12 +37,12 @@ int dense_block(skm_ctx* ctx, const float* d_x, size_t m, const float* d_c, cons
     for (size_t i0 = 0; i0 < m; i0 += sub) {
         const size_t mm = std::min(sub, m - i0);
         {
-            ScopedStage st(ctx, "search/blas");
+            ScopedStage st(ctx, "search/overflow/blas");
             SKM_TRY(launch_gemm_store(ctx, d_x + i0 * d, (int) mm, (int64_t) d, d_c, (int) k, (int64_t) d, (int) partial_d,
                                       (float*) ws_partial, (int64_t) ld, d_xnorm_p + i0, d_cnorm_p));
         }
         {
-            ScopedStage st(ctx, "search/pdx");
+            ScopedStage st(ctx, "search/overflow/pdx");
             SKM_TRY(launch_prune(ctx, (const float*) ws_partial, (int64_t) ld, d_x + i0 * d, (int) mm, d_c, d_pdx, d_aux,
                                  (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_idx + i0, d_dist + i0,
                                  d_counts + i0, d_stage));
@@ -88,16 +89,15 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     if (h_out_stage_pairs) SKM_TRY(skm_fill_u32(ctx, d_stage, 0u, 2 * (n_hblocks + 2)));
     unsigned long long* stage_arg = h_out_stage_pairs ? d_stage : nullptr;
 
-    // Per-chunk scalars: best0, thr0, candidate counts, overflow ids, overflow counter.
+    // Overflow ids of the whole call, then per-chunk scalars: best0, thr0, candidate counts.
     void* ws_chunk = nullptr;
-    SKM_TRY(workspace(ctx, 2, cn * (3 * sizeof(uint32_t) + sizeof(uint64_t)) + 256, &ws_chunk));
+    SKM_TRY(workspace(ctx, 2, n * sizeof(uint64_t) + cn * 3 * sizeof(uint32_t) + 256, &ws_chunk));
     uint64_t* d_over_ids = (uint64_t*) ws_chunk;
-    float* d_best0 = (float*) (d_over_ids + cn);
+    float* d_best0 = (float*) (d_over_ids + n);
     float* d_thr0 = d_best0 + cn;
     uint32_t* d_cand_count = (uint32_t*) (d_thr0 + cn);
     uint32_t* d_n_over = d_cand_count + cn;
-    void* h_pin = nullptr;
-    SKM_TRY(pinned(ctx, 64, &h_pin));
+    SKM_TRY(skm_fill_u32(ctx, d_n_over, 0u, 1));
 
     for (size_t i0 = 0; i0 < n; i0 += chunk) {
         const size_t m = std::min(chunk, n - i0);
@@ -108,43 +108,43 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
             ScopedStage st(ctx, "search/seed");
             SKM_TRY(launch_seed_distance(ctx, xc, d_c, d_inout_idx + i0, (int) m, (int) d, d_ratios, (int) partial_d,
                                          d_best0, d_thr0));
-            SKM_TRY(skm_fill_u32(ctx, d_cand_count, 0u, m));
-            SKM_TRY(skm_fill_u32(ctx, d_n_over, 0u, 1));
         }
         {
             ScopedStage st(ctx, "search/blas");
             SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
                                            d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
         }
-        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, d_over_ids, d_n_over));
-        SKM_HIP_TRY(hipMemcpyAsync(h_pin, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over));
         {
             ScopedStage st(ctx, "search/pdx");
             SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
                                       (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
                                       d_out_dist + i0, d_counts + i0, stage_arg));
         }
-        SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-        const uint32_t n_over = *(volatile uint32_t*) h_pin;
-        if (n_over > 0) {
-            // Dense redo of the overflowed points: gather them, run the dense pair, scatter the results back.
-            ScopedStage st(ctx, "search/overflow");
-            const size_t mo = n_over;
-            void* ws_o = nullptr;
-            SKM_TRY(workspace(ctx, 3, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
-            float* xo = (float*) ws_o;
-            float* xnorm_o = xo + mo * d;
-            uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
-            float* dist_o = (float*) (idx_o + align_up(mo, 64));
-            uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
-            SKM_TRY(skm_gather_rows(ctx, xc, d, d_over_ids, mo, xo, d_xnorm_p + i0, xnorm_o));
-            SKM_TRY(launch_gather_u32(ctx, d_inout_idx + i0, d_over_ids, (int) mo, idx_o));
-            SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p,
-                                idx_o, dist_o, cnt_o, stage_arg));
-            SKM_TRY(launch_scatter_u32(ctx, idx_o, d_over_ids, (int) mo, d_inout_idx + i0));
-            SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_over_ids, (int) mo, (uint32_t*) (d_out_dist + i0)));
-            SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_over_ids, (int) mo, d_counts + i0));
-        }
+    }
+    // Points whose list overflowed (loose seeds, or points with no centroid nearby): one dense redo for
+    // all of them: gather, dense partial distances + dense pruning, scatter the results back.
+    void* h_pin = nullptr;
+    SKM_TRY(pinned(ctx, 64, &h_pin));
+    SKM_HIP_TRY(hipMemcpyAsync(h_pin, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    const size_t mo = *(volatile uint32_t*) h_pin;
+    if (mo > 0) {
+        ScopedStage st(ctx, "search/overflow");
+        void* ws_o = nullptr;
+        SKM_TRY(workspace(ctx, 3, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
+        float* xo = (float*) ws_o;
+        float* xnorm_o = xo + mo * d;
+        uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
+        float* dist_o = (float*) (idx_o + align_up(mo, 64));
+        uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
+        SKM_TRY(skm_gather_rows(ctx, d_x, d, d_over_ids, mo, xo, d_xnorm_p, xnorm_o));
+        SKM_TRY(launch_gather_u32(ctx, d_inout_idx, d_over_ids, (int) mo, idx_o));
+        SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p, idx_o,
+                            dist_o, cnt_o, stage_arg));
+        SKM_TRY(launch_scatter_u32(ctx, idx_o, d_over_ids, (int) mo, d_inout_idx));
+        SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_over_ids, (int) mo, (uint32_t*) d_out_dist));
+        SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_over_ids, (int) mo, d_counts));
     }
     if (h_out_not_pruned) {
         double total = 0.0;

@@ -94,7 +94,7 @@ def test_assign_full_chunked_by_workspace_limit(capi, ctx, oracle):
         C2 = np.concatenate([C, g.standard_normal((40000, 96)).astype(np.float32) + 50.0])
         got = _assign_full(capi, ctx, np.tile(X, (5, 1)), C2)
     finally:
-        capi.check(ctx.lib.skm_ctx_set_workspace_limit(ctx.handle, 4 << 30))
+        capi.check(ctx.lib.skm_ctx_set_workspace_limit(ctx.handle, 24 << 30))
     assert np.array_equal(got[0][:3000], ref[0])
     assert np.array_equal(got[0][3000:6000], ref[0])
 
