@@ -163,6 +163,16 @@ int skm_synth_gaussian_mixture(skm_ctx* ctx, float* d_out, size_t n, size_t d, s
                                uint32_t n_centers, uint32_t center_seed, uint32_t point_seed,
                                float center_sigma, float noise_sigma, float decay_exponent, int normalize);
 
+/* Same kind of utility for the other benchmark shapes: a two-level mixture (n_coarse coarse centres,
+ * n_fine fine centres split evenly among them: x = coarse + fine_sigma * fine + noise_sigma * noise)
+ * and low-intrinsic-dimension rows with heavy tails (x = A z + noise_scale * Student-t(3), z ~ N(0, I_rank),
+ * A a fixed d x rank Gaussian map); rows are L2-normalised. */
+int skm_synth_two_level_mixture(skm_ctx* ctx, float* d_out, size_t n, size_t d, size_t row_offset,
+                                uint32_t n_coarse, uint32_t n_fine, uint32_t seed, float fine_sigma,
+                                float noise_sigma);
+int skm_synth_low_rank(skm_ctx* ctx, float* d_out, size_t n, size_t d, size_t row_offset, uint32_t rank,
+                       uint32_t seed, float noise_scale);
+
 #ifdef __cplusplus
 }
 #endif

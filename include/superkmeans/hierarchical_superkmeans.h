@@ -121,10 +121,16 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
                  hierarchical_config.use_blas_only, /*first_iteration_exact=*/true,
                  hierarchical_iteration_stats.mesoclustering_iteration_stats, hierarchical_config.early_termination);
 
-        // Sizes as left by the last consolidation, assignments of the last search.
-        mesoclusters_sizes.assign(this->cluster_sizes.get(), this->cluster_sizes.get() + n_mesoclusters);
+        // Assignments of the last search and the number of points they give every mesocluster.
+        // The reference takes the sizes from cluster_sizes, which SplitClusters has already edited when
+        // a mesocluster was empty in the last iteration (hierarchical_superkmeans.h:262-286); its
+        // partition of the points is then inconsistent with the assignments.  Here the sizes are
+        // recounted from the assignments, which is identical whenever no such split happened; an
+        // empty mesocluster simply receives no fine clusters.
         mesoclusters_assignments.resize(total_samples);
         this->d_assignments.Download(mesoclusters_assignments.data(), total_samples);
+        mesoclusters_sizes.assign(n_mesoclusters, 0u);
+        for (size_t i = 0; i < total_samples; ++i) mesoclusters_sizes[mesoclusters_assignments[i]]++;
 
         // Point ids grouped by mesocluster, ascending inside each group (counting sort).
         std::vector<uint64_t> indices_flat(total_samples);
@@ -132,17 +138,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         for (size_t m = 0; m < n_mesoclusters; ++m) offsets[m + 1] = offsets[m] + mesoclusters_sizes[m];
         {
             std::vector<size_t> cursor(offsets.begin(), offsets.end() - 1);
-            for (size_t i = 0; i < total_samples; ++i) {
-                const size_t m = mesoclusters_assignments[i];
-                if (cursor[m] >= offsets[m + 1]) {
-                    // Sizes were altered by a cluster split in the last mesoclustering iteration and no
-                    // longer describe the assignments; the reference indexes out of range here.
-                    throw std::runtime_error(
-                        "mesocluster sizes are inconsistent with assignments (a mesocluster was split in the "
-                        "last mesoclustering iteration)");
-                }
-                indices_flat[cursor[m]++] = i;
-            }
+            for (size_t i = 0; i < total_samples; ++i) indices_flat[cursor[mesoclusters_assignments[i]]++] = i;
         }
         dbuf<uint64_t> d_indices(ctx, total_samples);
         d_indices.Upload(indices_flat.data(), total_samples);

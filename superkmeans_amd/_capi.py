@@ -59,6 +59,9 @@ _PROTOTYPES = {
         c_int,
         [c_void_p, _F, c_size_t, c_size_t, c_size_t, c_uint32, c_uint32, c_uint32, c_float, c_float, c_float, c_int],
     ),
+    "skm_synth_two_level_mixture": (
+        c_int, [c_void_p, _F, c_size_t, c_size_t, c_size_t, c_uint32, c_uint32, c_uint32, c_float, c_float]),
+    "skm_synth_low_rank": (c_int, [c_void_p, _F, c_size_t, c_size_t, c_size_t, c_uint32, c_uint32, c_float]),
     # include/skm_kmeans.h
     "skm_kmeans_default_config": (None, [c_void_p, c_int]),
     "skm_kmeans_create": (c_int, [c_size_t, c_size_t, c_void_p, c_int, POINTER(c_void_p)]),
