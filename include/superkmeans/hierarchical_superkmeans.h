@@ -109,8 +109,9 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         // ---- phase 1: mesoclustering over all samples ----
         if (hierarchical_config.verbose)
             std::cout << "\n=== PHASE 1: MESOCLUSTERING (k=" << n_mesoclusters << " clusters) ===" << std::endl;
-        this->GenerateCentroids(data, total_samples, n_mesoclusters, rotate, on_device);
+        // Rotation first: it runs on the device while the host draws the initial mesocluster centroids.
         const float* data_to_cluster = this->SampleAndRotateVectors(data, n, total_samples, rotate, on_device);
+        this->GenerateCentroids(data, total_samples, n_mesoclusters, rotate, on_device);
         this->RotateOrCopy(this->horizontal_centroids.get(), this->prev_centroids.get(), n_mesoclusters, rotate);
         hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, d, this->data_norms.get()));
         // Full norms of every sample, kept for the fine phase whose first iteration is always exact.
@@ -249,7 +250,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         for (size_t ci = 0; ci < k; ci++) {
             if (sizes[ci] != 0) continue;
             size_t cj;
-            for (cj = 0; true; cj = (cj + 1) % k) {
+            for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
                 float p = (sizes[cj] - 1.0f) / static_cast<float>(n_samples_ - k);
                 float r = std::uniform_real_distribution<float>(0, 1)(rng);
                 if (r < p) break;

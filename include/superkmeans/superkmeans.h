@@ -337,8 +337,10 @@ class SuperKMeans {
         }
 
         const bool rotate = !config.data_already_rotated;
-        GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
+        // The rotation of the training matrix is queued first so that it runs on the device while the host
+        // draws the initial centroids; the two steps share no state (each seeds its own mt19937).
         const float* data_to_cluster = SampleAndRotateVectors(data, n, n_samples, rotate, on_device);
+        GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
         // prev_centroids <- rotated initial centroids; horizontal_centroids still holds the raw rows.
         RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
         hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, d, data_norms.get()));
@@ -476,7 +478,7 @@ class SuperKMeans {
         for (size_t ci = 0; ci < k; ci++) {
             if (cluster_sizes[ci] != 0) continue;
             size_t cj;
-            for (cj = 0; true; cj = (cj + 1) % k) {
+            for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
                 float p = (cluster_sizes[cj] - 1.0) / (float) (n_samples_ - k);
                 float r = std::uniform_real_distribution<float>(0, 1)(rng);
                 if (r < p) break;
@@ -677,7 +679,7 @@ class SuperKMeans {
         }
         training_data.Reset(ctx, n_samples_ * d);
         pruner->Rotate(d_raw, training_data.get(), n_samples_);
-        hip::Check(skm_sync(ctx));  // `staged` is released on return
+        if (staged.get() != nullptr) hip::Check(skm_sync(ctx));  // `staged` is released on return
         return training_data.get();
     }
 

@@ -217,12 +217,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     const int ld_row = tid >> 3;
     const int ld_k = (tid & 7) * 4;
 
+    // Row offsets of the four point rows this thread stages (clamped: padding points never pass).
     const float* b_rows[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         int rb = tn * GEMM_TN + ld_row + 32 * p;
         rb = rb < g.N ? rb : g.N - 1;
-        b_rows[p] = g.B + (int64_t) rb * g.ldb;
+        b_rows[p] = g.B + (int64_t) rb * g.ldb + ld_k;
     }
     // The two points of this lane.
     int pt[2];
@@ -235,34 +236,45 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
         thr[nb] = valid ? thr0[pt[nb]] : -3.0e38f;  // nothing passes for padding columns
     }
 
-    const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;
-    const int nk_full = VEC ? g.K / GEMM_BK : 0;
+    uint2* list[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) list[nb] = cand + (int64_t) (pt[nb] < g.N ? pt[nb] : 0) * cap;
+
+    const int nk_full = VEC ? g.K / GEMM_BK : 0;       // slices fetched without guards
+    const int n_full_steps = g.K / GEMM_BK;            // slices whose 32 columns all hold data
+    const bool has_tail = (g.K % GEMM_BK) != 0;
+    const int tail_groups = (g.K % GEMM_BK + 7) / 8;
     floatx4 ra[4], rb[4];
     float cn_next = 0.0f;
 
-    // Requests operand slice `kt` of centroid tile `tm` (and that tile's norms when kt == 0).
-    auto request = [&](int tm, int kt) {
-        const int k0 = kt * GEMM_BK + ld_k;
-        if (kt < nk_full) {
+    // Operand slice `kt` of centroid tile `tm`, every column in range (no guard, loads issued back to back).
+    auto request_full = [&](int tm, int kt) {
+        const int k0 = kt * GEMM_BK;
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                int r = tm * GEMM_TM + ld_row + 32 * p;
-                r = r < g.M ? r : g.M - 1;
-                ra[p] = load_k4<VEC, false>(g.A + (int64_t) r * g.lda, k0, g.K);
-                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
-            }
-        } else {
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                int r = tm * GEMM_TM + ld_row + 32 * p;
-                r = r < g.M ? r : g.M - 1;
-                ra[p] = load_k4<VEC, true>(g.A + (int64_t) r * g.lda, k0, g.K);
-                rb[p] = load_k4<VEC, true>(b_rows[p], k0, g.K);
-            }
+        for (int p = 0; p < 4; ++p) {
+            int r = tm * GEMM_TM + ld_row + 32 * p;
+            r = r < g.M ? r : g.M - 1;
+            ra[p] = load_k4<VEC, false>(g.A + (int64_t) r * g.lda + ld_k, k0, g.K);
+            rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
         }
-        if (kt == 0 && tid < GEMM_TM) {
+    };
+    // Same with columns at or past K read as zero (trailing slice; every slice of the scalar path).
+    auto request_guarded = [&](int tm, int kt) {
+        const int k0 = kt * GEMM_BK + ld_k;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            int r = tm * GEMM_TM + ld_row + 32 * p;
+            r = r < g.M ? r : g.M - 1;
+            ra[p] = load_k4<VEC, true>(g.A + (int64_t) r * g.lda, k0, g.K);
+            rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0, g.K);
+        }
+    };
+    // First slice of tile `tm` plus that tile's centroid norms (rows past M get a norm nothing passes with).
+    auto request_first = [&](int tm) {
+        if (nk_full > 0) request_full(tm, 0); else request_guarded(tm, 0);
+        if (tid < GEMM_TM) {
             const int m = tm * GEMM_TM + tid;
-            cn_next = m < g.M ? cnorm[m] : 0.0f;
+            cn_next = m < g.M ? cnorm[m] : 3.0e38f;
         }
     };
     const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
@@ -277,7 +289,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     };
 
     int cur = 0;
-    request(0, 0);
+    request_first(0);
     publish(0);
     if (tid < GEMM_TM) {
         cn_s[tid] = cn_next;
@@ -286,6 +298,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     __syncthreads();
 
     const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
+    const int a_frag = (wm * 64) * GEMM_LDS_STRIDE + frag_off;
+    const int b_frag = (wn * 64) * GEMM_LDS_STRIDE + frag_off;
     for (int tm = 0; tm < g.tiles_m; ++tm) {
         WaveAcc acc;
 #pragma unroll
@@ -295,53 +309,80 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
         const bool next_tile = (tm + 1) < g.tiles_m;
-        for (int kt = 0; kt < nk; ++kt) {
-            const bool inner = (kt + 1) < nk;
-            if (inner) {
-                request(tm, kt + 1);
-            } else if (next_tile) {
-                request(tm + 1, 0);
-            }
-            const float* as = As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off;
-            const float* bs = Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off;
-            const int k_left = g.K - kt * GEMM_BK;
-            if (k_left >= GEMM_BK) {
-                mfma_step_full(as, bs, acc);
-            } else {
-                mfma_step_tail(as, bs, acc, (k_left + 7) / 8);
-            }
-            if (inner) {
+
+        // Full slices whose successor is a full slice of the same tile: the hot loop, free of guards.
+        for (int kt = 0; kt + 1 < nk_full; ++kt) {
+            request_full(tm, kt + 1);
+            __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs they overlap with
+            mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
+            __builtin_amdgcn_sched_barrier(0);
+            publish(cur ^ 1);
+            __syncthreads();
+            cur ^= 1;
+        }
+        // Scalar path: every slice is fetched with guards.
+        if (!VEC) {
+            for (int kt = 0; kt + 1 < n_full_steps; ++kt) {
+                request_guarded(tm, kt + 1);
+                mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
                 publish(cur ^ 1);
                 __syncthreads();
                 cur ^= 1;
             }
         }
+        // Last full slice: its successor is the trailing partial slice or the next tile's first slice.
+        if (n_full_steps > 0) {
+            if (has_tail) {
+                request_guarded(tm, n_full_steps);
+            } else if (next_tile) {
+                request_first(tm + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
+            if (has_tail) {
+                publish(cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+        if (has_tail) {
+            if (next_tile) request_first(tm + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc, tail_groups);
+        }
 
         // ---- epilogue of tile tm: first pruning test, candidates appended to the per-point lists ----
         const float* cns = cn_s + (tm & 1) * GEMM_TM + wm * 64;
         const int m0 = tm * GEMM_TM + wm * 64;
+        // Passing pairs are rare (a fraction of a percent).  The outcome of the 32 tests of one point is
+        // collected in a per-lane bit mask (the sign of v - thr is shifted in, so a test costs four vector
+        // instructions and no scalar dependency); lanes with an empty mask skip the append.
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
-            uint32_t pass = 0;  // bit (mb * 16 + r)
+            uint32_t pass = 0;  // element (mb, r) lands in bit 31 - (mb * 16 + r)
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int ml = acc_row(mb, r, lane);
-                    const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn[nb]) + cns[ml];
-                    acc.v[mb][nb][r] = v;
-                    if (m0 + ml < g.M && v < thr[nb]) pass |= 1u << (mb * 16 + r);
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const floatx4 c4 = *reinterpret_cast<const floatx4*>(&cns[acc_row(mb, r4 * 4, lane)]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int r = r4 * 4 + j;
+                        const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn[nb]) + c4[j];
+                        acc.v[mb][nb][r] = v;
+                        // v < thr  <=>  the IEEE difference v - thr carries a set sign bit.
+                        pass = __builtin_amdgcn_alignbit(pass, __float_as_uint(v - thr[nb]), 31);
+                    }
                 }
             if (pass) {
                 uint32_t slot = atomicAdd(&cnt_s[wn * 64 + acc_col(nb, lane)], (uint32_t) __popc(pass));
-                uint2* list = cand + (int64_t) pt[nb] * cap;
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        if (pass & (1u << (mb * 16 + r))) {
+                        if (pass & (0x80000000u >> (mb * 16 + r))) {
                             if (slot < cap)
-                                list[slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
+                                list[nb][slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
                             ++slot;
                         }
                     }

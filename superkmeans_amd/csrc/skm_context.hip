@@ -157,17 +157,18 @@ int skm_ctx_create(int device, skm_ctx** out_ctx) {
 
 int skm_ctx_destroy(skm_ctx* ctx) {
     if (!ctx) return SKM_OK;
-    hipSetDevice(ctx->device);
-    hipStreamSynchronize(ctx->stream);
+    // Teardown keeps going after a failure so that every resource gets its release call.
+    (void) hipSetDevice(ctx->device);
+    (void) hipStreamSynchronize(ctx->stream);
     for (auto& iv : ctx->pending) {
-        hipEventDestroy(iv.start);
-        hipEventDestroy(iv.stop);
+        (void) hipEventDestroy(iv.start);
+        (void) hipEventDestroy(iv.stop);
     }
-    for (auto e : ctx->event_pool) hipEventDestroy(e);
+    for (auto e : ctx->event_pool) (void) hipEventDestroy(e);
     for (int i = 0; i < 4; ++i)
-        if (ctx->ws[i]) hipFree(ctx->ws[i]);
-    if (ctx->h_pinned) hipHostFree(ctx->h_pinned);
-    hipStreamDestroy(ctx->stream);
+        if (ctx->ws[i]) (void) hipFree(ctx->ws[i]);
+    if (ctx->h_pinned) (void) hipHostFree(ctx->h_pinned);
+    (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     return SKM_OK;
 }
