@@ -29,6 +29,15 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBPS = 8000.0
 
 
+# L2 <-> fabric bytes of one gemm_argmin_kernel launch, from two rocprofv3 --pmc passes (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch) scaled by what the same counters read for a copy kernel of known size
+# (FETCH_SIZE x 1.943, WRITE_SIZE x 1.000); counters cannot be read from inside this process, so the figure is
+# kept per workload shape (n, d, k) and is null for shapes that were not profiled.
+MEASURED_TRAFFIC_BYTES = {
+    (1_000_000, 1024, 10_000): int((88_194_781 * 1.943 + 1_226_562) * 1024),
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,7 +179,7 @@ def main():
     achieved = flops_per_launch / (gemm_avg_ms * 1e-3) / 1e12 if gemm_avg_ms > 0 else 0.0
     roofline = {"kernel": "gemm_argmin_kernel", "bound": "mfma", "achieved": round(achieved, 2),
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": None, "avg_launch_ms": round(gemm_avg_ms, 3), "flops_per_launch": flops_per_launch}
+                "traffic": MEASURED_TRAFFIC_BYTES.get((n, d, k)), "avg_launch_ms": round(gemm_avg_ms, 3), "flops_per_launch": flops_per_launch}
     gpu_assign = dOut.download()
 
     # ---- CPU baseline: the oracle on a bounded prefix of the same points ----

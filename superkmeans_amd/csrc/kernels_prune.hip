@@ -86,6 +86,9 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
     const int d = a.d, V = a.vertical_d, dp = a.partial_d;
     const int H = d - V;
     const int n_hblocks = H / SKM_H_DIM_SIZE;
+    // Accounting counters come in SKM_ACCT_COPIES striped copies (summed by the host) so that the
+    // atomics of concurrently running workgroups spread over many addresses.
+    unsigned long long* acct = a.stage_pairs ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
     const float* xq = a.x + (int64_t) p * d;
     const int sub = lane & 15;   // lane within a 16-lane group
     const int grp = lane >> 4;   // which of the 4 survivors handled per step
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             cnt += __popcll(mask);
         }
         not_pruned_total += (uint32_t) cnt;
-        if (a.stage_pairs && lane == 0 && cnt) atomicAdd(&a.stage_pairs[0], (unsigned long long) cnt);
+        if (acct && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
         // Only survivor is the incumbent: nothing to do (pdxearch.h:140-143).
         if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
         if (cnt == 0) continue;
@@ -148,7 +151,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
         const float* chunk = a.pdx + (int64_t) base * d;
         int dims_seen = dp;
         for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
-            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + hb], (unsigned long long) cnt);
+            if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
             const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
             const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
             float4 xv;
@@ -183,7 +186,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
 
         // ---- remaining vertical dimensions [d', V) from the dense auxiliary copy (pdxearch.h:183-216) ----
         if (cnt > 0 && dp < V) {
-            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + n_hblocks], (unsigned long long) cnt);
+            if (acct && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
             const int left = V - dp;
             for (int s0 = 0; s0 < cnt; s0 += 4) {
                 const int s = s0 + grp;
@@ -313,6 +316,9 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
     float* acc = s_acc[wave];
     const int d = a.d, V = a.vertical_d, dp = a.partial_d;
     const int n_hblocks = (d - V) / SKM_H_DIM_SIZE;
+    // Accounting counters come in SKM_ACCT_COPIES striped copies (summed by the host) so that the
+    // atomics of concurrently running workgroups spread over many addresses.
+    unsigned long long* acct = a.stage_pairs ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
     const float* xq = a.x + (int64_t) p * d;
     const uint2* list = a.cand + (int64_t) p * a.cap;
     const int sub = lane & 15, grp = lane >> 4;
@@ -371,14 +377,14 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
         }
         jb = next_jb;
         not_pruned_total += (uint32_t) cnt;
-        if (a.stage_pairs && lane == 0 && cnt) atomicAdd(&a.stage_pairs[0], (unsigned long long) cnt);
+        if (acct && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
         if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
         if (cnt == 0) continue;
 
         const float* chunk = a.pdx + (int64_t) base * d;
         int dims_seen = dp;
         for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
-            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + hb], (unsigned long long) cnt);
+            if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
             const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
             const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
             float4 xv;
@@ -411,7 +417,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
             cnt = compact_survivors(pos, acc, cnt, thr, lane);
         }
         if (cnt > 0 && dp < V) {
-            if (a.stage_pairs && lane == 0) atomicAdd(&a.stage_pairs[1 + n_hblocks], (unsigned long long) cnt);
+            if (acct && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
             const int left = V - dp;
             for (int s0 = 0; s0 < cnt; s0 += 4) {
                 const int s = s0 + grp;

@@ -93,6 +93,8 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
 int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, uint32_t* out_idx,
                           float* out_dist);
 
+// Number of striped copies of the per-stage accounting counters (each n_hblocks + 2 entries long).
+constexpr int SKM_ACCT_COPIES = 64;
 int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
                  const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
                  int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,

@@ -83,10 +83,10 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     const size_t cn = std::min(chunk, n);
 
     void* ws_counts = nullptr;
-    SKM_TRY(workspace(ctx, 1, n * sizeof(uint32_t) + (n_hblocks + 2) * sizeof(unsigned long long) + 64, &ws_counts));
+    SKM_TRY(workspace(ctx, 1, n * sizeof(uint32_t) + SKM_ACCT_COPIES * (n_hblocks + 2) * sizeof(unsigned long long) + 64, &ws_counts));
     unsigned long long* d_stage = (unsigned long long*) ws_counts;
-    uint32_t* d_counts = (uint32_t*) (d_stage + n_hblocks + 2);
-    if (h_out_stage_pairs) SKM_TRY(skm_fill_u32(ctx, d_stage, 0u, 2 * (n_hblocks + 2)));
+    uint32_t* d_counts = (uint32_t*) (d_stage + SKM_ACCT_COPIES * (n_hblocks + 2));
+    if (h_out_stage_pairs) SKM_TRY(skm_fill_u32(ctx, d_stage, 0u, 2 * SKM_ACCT_COPIES * (n_hblocks + 2)));
     unsigned long long* stage_arg = h_out_stage_pairs ? d_stage : nullptr;
 
     // Overflow ids of the whole call, then per-chunk scalars: best0, thr0, candidate counts.
@@ -152,11 +152,11 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         *h_out_not_pruned = (uint64_t) total;
     }
     if (h_out_stage_pairs) {
-        std::vector<unsigned long long> tmp(n_hblocks + 2);
+        std::vector<unsigned long long> tmp(SKM_ACCT_COPIES * (n_hblocks + 2));
         SKM_HIP_TRY(hipMemcpyAsync(tmp.data(), d_stage, tmp.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost,
                                    ctx->stream));
         SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-        for (size_t s = 0; s < tmp.size(); ++s) h_out_stage_pairs[s] = tmp[s];
+        for (size_t s = 0; s < tmp.size(); ++s) h_out_stage_pairs[s % (n_hblocks + 2)] += tmp[s];
     }
     return SKM_OK;
 }
