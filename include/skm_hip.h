@@ -5,7 +5,7 @@
  * BLAS sgemm_, OpenMP loops and AVX/NEON kernels.  Each entry point below
  * replaces one of those CPU routines with hand-written HIP kernels; the cited
  * file:line is the reference routine it stands in for (paths relative to the
- * reference's include/superkmeans/).  Host C++ (include/superkmeans/*.h) and
+ * reference's include/superkmeans/).  Host C++ (the headers under include/superkmeans) and
  * the language bindings call only this header; no HIP type crosses it.
  *
  * Conventions
@@ -152,6 +152,20 @@ int skm_gather_rows(skm_ctx* ctx, const float* d_x, size_t d, const uint64_t* d_
  * out[index[j]] = local[j] + offset. */
 int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_t* d_local, size_t m,
                             uint32_t offset, uint32_t* d_out);
+/* BatchComputer::FindKNearestNeighbors (batch_computers.h:191-274): for every row of x the k rows of
+ * y with the smallest -2 x.y + ||x||^2 + ||y||^2, ordered by (distance, index), y taken in batches of
+ * 1024 rows: entries kept from earlier batches compete with their distance clamped at 0, the result
+ * is clamped at 0; slots beyond n_y hold {FLT_MAX, 0xffffffff}.  k <= 1024.
+ * d_out_idx / d_out_dist: n_x * k. */
+int skm_knn(skm_ctx* ctx, const float* d_x, size_t n_x, const float* d_y, size_t n_y, size_t d,
+            const float* d_xnorm, const float* d_ynorm, size_t k, uint32_t* d_out_idx, float* d_out_dist);
+/* Inner loops of SuperKMeans::ComputeRecall (superkmeans.h:1064-1082): h_out_hits[q] = how many of
+ * query q's objective_k ground-truth neighbours (row ids into the training sample) are assigned to one
+ * of the query's `explore` promising centroids.  explore <= 1024.  The caller forms
+ * sum_q (float) hits[q] / objective_k in query order, then divides by n_queries. */
+int skm_recall_hits(skm_ctx* ctx, const uint32_t* d_gt, const uint32_t* d_promising,
+                    const uint32_t* d_assignments, size_t n_assignments, size_t n_queries,
+                    size_t objective_k, size_t explore, uint32_t* h_out_hits);
 
 /* Benchmark / test utility: seeded Gaussian-mixture rows generated in device memory.  Row i (logical
  * index row_offset + local row) is  s_j * (center_sigma * g(center_seed, u_i, j) + noise_sigma *

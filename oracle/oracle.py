@@ -191,6 +191,30 @@ def find_nn(x, y, norms_x=None, norms_y=None):
     return knn, dist
 
 
+def find_knn(x, y, k, norms_x=None, norms_y=None):
+    """FindKNearestNeighbors (batch_computers.h:191-274): (indices, distances), each (n_x, k)."""
+    x, y = f32(x), f32(y)
+    nx = norms(x) if norms_x is None else f32(norms_x)
+    ny = norms(y) if norms_y is None else f32(norms_y)
+    knn = np.zeros((x.shape[0], k), dtype=np.uint32)
+    dist = np.empty((x.shape[0], k), dtype=np.float32)
+    lib = load()
+    lib.oracle_find_knn(_fp(x), _fp(y), c_size_t(x.shape[0]), c_size_t(y.shape[0]), c_size_t(x.shape[1]), _fp(nx),
+                        _fp(ny), c_size_t(k), _fp(knn), _fp(dist))
+    return knn, dist
+
+
+def recall_from_lists(gt, promising, assignments):
+    """Recall loop of ComputeRecall (superkmeans.h:1059-1086) on (n_q, objective_k) / (n_q, explore) lists."""
+    gt = np.ascontiguousarray(gt, dtype=np.uint32)
+    promising = np.ascontiguousarray(promising, dtype=np.uint32)
+    assignments = np.ascontiguousarray(assignments, dtype=np.uint32)
+    lib = load()
+    lib.oracle_recall_from_lists.restype = ctypes.c_float
+    return float(lib.oracle_recall_from_lists(_fp(gt), _fp(promising), _fp(assignments), c_size_t(gt.shape[0]),
+                                              c_size_t(gt.shape[1]), c_size_t(promising.shape[1])))
+
+
 def find_nn_pruned(x, y, prev_assign, partial_d, ratio_table, accounting=False):
     """FindNearestNeighborWithPruning on rotated x and centroids y; returns (assign, dist, counts[, stage_pairs])."""
     x, y = f32(x), f32(y)

@@ -472,6 +472,29 @@ static void FindKNearestNeighbors(const float* x, const float* y, const size_t n
     }
 }
 
+// ---- superkmeans.h:1059-1086: recall@objective_k from the ground-truth and promising-centroid lists ----
+static float RecallFromLists(const uint32_t* gt_assignments, const uint32_t* promising_centroids,
+                             const uint32_t* assignments, const size_t n_queries, const size_t objective_k,
+                             const size_t centroids_to_explore) {
+    float sum_recall = 0.0f;
+    for (size_t i = 0; i < n_queries; ++i) {
+        size_t found_in_query = 0;
+        for (size_t j = 0; j < objective_k; ++j) {
+            uint32_t gt = gt_assignments[i * objective_k + j];
+            bool found = false;
+            for (size_t t = 0; t < centroids_to_explore; ++t) {
+                if (promising_centroids[i * centroids_to_explore + t] == assignments[gt]) {
+                    found = true;
+                    break;
+                }
+            }
+            if (found) ++found_in_query;
+        }
+        sum_recall += static_cast<float>(found_in_query) / static_cast<float>(objective_k);
+    }
+    return sum_recall / static_cast<float>(n_queries);
+}
+
 // ---- batch_computers.h:297-409 ----
 static void FindNearestNeighborWithPruning(const float* x, const float* y, const size_t n_x, const size_t n_y,
                                            const size_t d, const float* norms_x, const float* norms_y,
@@ -1102,23 +1125,8 @@ class KMeans {
         FindKNearestNeighbors(queries, horizontal_centroids.get(), n_queries, n_clusters, d, query_norms.get(),
                               centroid_norms.get(), centroids_to_explore, promising_centroids.get(),
                               recall_distances.get(), tmp_distances_buffer.get());
-        float sum_recall = 0.0f;
-        for (size_t i = 0; i < n_queries; ++i) {
-            size_t found_in_query = 0;
-            for (size_t j = 0; j < config.objective_k; ++j) {
-                uint32_t gt = gt_assignments[i * config.objective_k + j];
-                bool found = false;
-                for (size_t t = 0; t < centroids_to_explore; ++t) {
-                    if (promising_centroids[i * centroids_to_explore + t] == assignments[gt]) {
-                        found = true;
-                        break;
-                    }
-                }
-                if (found) ++found_in_query;
-            }
-            sum_recall += static_cast<float>(found_in_query) / static_cast<float>(config.objective_k);
-        }
-        return sum_recall / static_cast<float>(n_queries);
+        return RecallFromLists(gt_assignments.get(), promising_centroids.get(), assignments.get(), n_queries,
+                               config.objective_k, centroids_to_explore);
     }
 
     // superkmeans.h:1100-1142
@@ -1587,6 +1595,15 @@ void oracle_find_nn_pruned(const float* x, const float* y, size_t n_x, size_t n_
         for (size_t s = 0; s < acct.pairs.size(); ++s) stage_pairs[s] = acct.pairs[s];
 }
 
+void oracle_find_knn(const float* x, const float* y, size_t n_x, size_t n_y, size_t d, const float* norms_x,
+                     const float* norms_y, size_t k, uint32_t* out_knn, float* out_distances) {
+    std::vector<float> tmp(X_BATCH_SIZE * Y_BATCH_SIZE);
+    FindKNearestNeighbors(x, y, n_x, n_y, d, norms_x, norms_y, k, out_knn, out_distances, tmp.data());
+}
+float oracle_recall_from_lists(const uint32_t* gt, const uint32_t* promising, const uint32_t* assignments,
+                               size_t n_queries, size_t objective_k, size_t explore) {
+    return RecallFromLists(gt, promising, assignments, n_queries, objective_k, explore);
+}
 void oracle_brute_force(const float* x, const float* y, size_t n_x, size_t n_y, size_t d, uint32_t* out_knn,
                         double* out_distances, double* out_second) {
     BruteForce(x, y, n_x, n_y, d, out_knn, out_distances, out_second);

@@ -55,6 +55,8 @@ _PROTOTYPES = {
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),
+    "skm_knn": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_size_t, _F, _F, c_size_t, _F, _F]),
+    "skm_recall_hits": (c_int, [c_void_p, _F, _F, _F, c_size_t, c_size_t, c_size_t, c_size_t, c_void_p]),
     "skm_synth_gaussian_mixture": (
         c_int,
         [c_void_p, _F, c_size_t, c_size_t, c_size_t, c_uint32, c_uint32, c_uint32, c_float, c_float, c_float, c_int],
@@ -154,6 +156,10 @@ def load():
         fn.argtypes = args
     _lib = lib
     return lib
+
+
+# Return codes of the C ABI (include/skm_hip.h, include/skm_kmeans.h).
+SKM_OK, SKM_ERR_INVALID, SKM_ERR_HIP, SKM_ERR_NO_DEVICE, SKM_ERR_OOM, SKM_ERR_RUNTIME = 0, -1, -2, -3, -4, -5
 
 
 def check(rc):

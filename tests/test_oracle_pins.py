@@ -379,3 +379,53 @@ def test_assign_training_points_agreement(oracle, blobs):
     ch = kh.train(X)
     assert np.mean(kh.assign_training_points(X, ch) == kh.assign(X, ch)) >= 0.98
     assert len(np.unique(kh.assign(X, ch))) >= 0.95 * 300
+
+
+# ---- FindKNearestNeighbors (batch_computers.h:191-274), test shape of tests/test_distance_computers.cpp:201-262 ----
+@pytest.mark.parametrize("n_x,n_y,d,k", [(1000, 500, 128, 10), (64, 3000, 96, 100), (7, 5, 16, 10)])
+def test_find_knn_against_fp64_brute_force(oracle, n_x, n_y, d, k):
+    rng = np.random.default_rng(42)
+    x = rng.uniform(-10, 10, (n_x, d)).astype(np.float32)
+    y = rng.uniform(-10, 10, (n_y, d)).astype(np.float32)
+    knn, dist = oracle.find_knn(x, y, k)
+    d64 = ((x.astype(np.float64)[:, None, :] - y.astype(np.float64)[None, :, :]) ** 2).sum(-1)
+    order = np.argsort(d64, axis=1, kind="stable")[:, :k]
+    kk = min(k, n_y)
+    ref_d = np.take_along_axis(d64, order, axis=1)
+    # indices equal unless the two distances tie to 1e-4 relative; distances within 1e-4 (the reference's bars)
+    rel = np.abs(dist[:, :kk] - ref_d[:, :kk]) / np.maximum(ref_d[:, :kk], 1e-6)
+    assert rel.max() <= 1e-4
+    assert np.all((knn[:, :kk] == order[:, :kk]) | (rel <= 1e-4))
+    assert np.mean(knn[:, :kk] == order[:, :kk]) > 0.999
+    assert np.all(np.diff(dist[:, :kk], axis=1) >= 0)  # sorted
+    if kk < k:  # slots beyond n_y stay unfilled (:204-205, :265-268)
+        assert np.all(knn[:, kk:] == 0xFFFFFFFF) and np.all(dist[:, kk:] == np.finfo(np.float32).max)
+
+
+def test_find_knn_batches_ties_and_progressive_clamp(oracle):
+    # Hand-built: d = 1, queries and rows chosen so that every distance is exact in fp32.
+    # Rows 0..1023 form batch 0, rows 1024.. batch 1.  Query 0 sits at 0.
+    y = np.full((1030, 1), 100.0, dtype=np.float32)
+    y[5, 0], y[900, 0], y[1025, 0], y[1027, 0] = 3.0, -3.0, 3.0, 1.0  # distances 9, 9, 9, 1
+    x = np.zeros((1, 1), dtype=np.float32)
+    knn, dist = oracle.find_knn(x, y, 3)
+    # (distance, index) order: (1,1027), (9,5), (9,900); (9,1025) loses the tie on index
+    assert knn[0].tolist() == [1027, 5, 900] and dist[0].tolist() == [1.0, 9.0, 9.0]
+    # Progressive clamp: a negative raw distance is stored as 0 after its batch, so a smaller negative one
+    # of a later batch sorts in front of it although its raw value is larger.
+    x = np.ones((1, 1), dtype=np.float32)
+    y[1027, 0] = 2.0                                   # -2*2 + 1 + 4 = 1
+    ynorm = (y[:, 0] ** 2).astype(np.float32)          # rows at 100: -200 + 1 + 10000 = 9801
+    xnorm = np.ones(1, dtype=np.float32)
+    ynorm[5] = 3.0     # -2*3 + 1 + 3 = -2: a negative rounding residue, exaggerated
+    ynorm[1025] = 4.0  # -2*3 + 1 + 4 = -1
+    knn, dist = oracle.find_knn(x, y, 3, norms_x=xnorm, norms_y=ynorm)
+    assert knn[0].tolist() == [1025, 5, 1027] and dist[0].tolist() == [0.0, 0.0, 1.0]
+
+
+def test_recall_from_lists_by_hand(oracle):
+    # 2 queries, objective_k = 4, explore = 2; assignments of 6 sample rows.
+    assign = np.array([0, 1, 2, 2, 3, 1], dtype=np.uint32)
+    gt = np.array([[0, 1, 2, 3], [4, 5, 0, 1]], dtype=np.uint32)          # clusters [0,1,2,2] and [3,1,0,1]
+    promising = np.array([[2, 7], [1, 3]], dtype=np.uint32)                # hits: 2 of 4, 3 of 4
+    assert oracle.recall_from_lists(gt, promising, assign) == np.float32((np.float32(0.5) + np.float32(0.75)) / 2)
