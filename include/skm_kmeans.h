@@ -75,8 +75,10 @@ int skm_kmeans_destroy(skm_kmeans* km);
  * h_out_centroids receives k x d floats. */
 int skm_kmeans_train(skm_kmeans* km, const float* h_data, size_t n, const float* h_queries, size_t n_queries,
                      float* h_out_centroids);
-/* Same with d_data already in device memory (no counterpart in the reference). */
-int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, float* h_out_centroids);
+/* Same with d_data (and d_queries, when n_queries > 0 and queries are not sampled) already in device
+ * memory (no counterpart in the reference). */
+int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, const float* d_queries,
+                            size_t n_queries, float* h_out_centroids);
 
 /* Assign (superkmeans.h:346): exact nearest centroid of each of the n vectors. */
 int skm_kmeans_assign(skm_kmeans* km, const float* h_vectors, const float* h_centroids, size_t n_vectors,

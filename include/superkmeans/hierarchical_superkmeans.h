@@ -65,8 +65,11 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         return TrainHierarchical(data, n, n_queries, /*on_device=*/false);
     }
 
-    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n) {
-        return TrainHierarchical(d_data, n, 0, /*on_device=*/true);
+    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n,
+                                              const vector_value_t* d_queries = nullptr,
+                                              const size_t n_queries = 0) {
+        (void) d_queries;
+        return TrainHierarchical(d_data, n, n_queries, /*on_device=*/true);
     }
 
     static size_t GetNMesoclusters(const size_t n_clusters) {

@@ -139,8 +139,10 @@ class SuperKMeans {
     }
 
     /** Train for data that already lives in device memory of this object's context. */
-    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n) {
-        return TrainImpl(d_data, n, nullptr, 0, /*on_device=*/true);
+    std::vector<centroid_value_t> TrainDevice(const vector_value_t* d_data, const size_t n,
+                                              const vector_value_t* d_queries = nullptr,
+                                              const size_t n_queries = 0) {
+        return TrainImpl(d_data, n, d_queries, n_queries, /*on_device=*/true);
     }
 
     /** Exact nearest-centroid assignment; vectors and centroids must be in the same space. */
@@ -319,10 +321,6 @@ class SuperKMeans {
         if (n_queries > 0 && queries == nullptr && !config.sample_queries) {
             throw std::invalid_argument("Queries must be provided if n_queries > 0 and sample_queries is false");
         }
-        if (n_queries > 0) {
-            throw std::runtime_error(
-                "recall-based early termination (queries) is not available in the HIP backend yet");
-        }
         n_samples = GetNVectorsToSample(n, n_clusters);
         if (n_samples < n_clusters) {
             throw std::runtime_error(
@@ -344,6 +342,8 @@ class SuperKMeans {
         // prev_centroids <- rotated initial centroids; horizontal_centroids still holds the raw rows.
         RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
         hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, d, data_norms.get()));
+        n_tracked_queries = 0;
+        if (n_queries) PrepareQueries(data_to_cluster, queries, n_queries, on_device);
 
         const bool always_gemm_only = d < DIMENSION_THRESHOLD_FOR_PRUNING || config.use_blas_only ||
                                       n_clusters <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;
@@ -358,7 +358,8 @@ class SuperKMeans {
             }
             RunIteration(use_gemm_only, data_to_cluster, n_samples, n_clusters, iter_idx,
                          use_gemm_only && iter_idx == 0, iteration_stats);
-            if (config.early_termination && ShouldStopEarly(false, best_recall, iters_without_improvement, iter_idx)) {
+            if (config.early_termination &&
+                ShouldStopEarly(n_queries > 0, best_recall, iters_without_improvement, iter_idx)) {
                 break;
             }
         }
@@ -420,6 +421,10 @@ class SuperKMeans {
         ConsolidateCentroids(n_samples_, k);
         ComputeCost(n_samples_);
         ComputeShift(k);
+        if (n_tracked_queries) {
+            hip::Check(skm_norms(ctx, horizontal_centroids.get(), k, d, d, centroid_norms.get()));
+            recall = ComputeRecall(n_samples_, k);
+        }
 
         SuperKMeansIterationStats stats;
         stats.iteration = iter_idx + 1;
@@ -517,6 +522,84 @@ class SuperKMeans {
         double s = 0.0;
         hip::Check(skm_shift(ctx, horizontal_centroids.get(), prev_centroids.get(), k, d, &s));
         shift = static_cast<float>(s);
+    }
+
+    /**
+     * Query set-up of Train (reference superkmeans.h:243-274): the rotated queries (given, or drawn from the
+     * training sample with the first n_queries entries of a mt19937(seed) shuffle of [0, n_samples)), their
+     * norms, and for every query its objective_k nearest training rows (GetGTAssignmentsAndDistances,
+     * superkmeans.h:1010-1031).  data_norms must hold full-dimension norms, as they do at this point of Train.
+     * The reference's draw reuses the member that maps sampled rows back to the input, which breaks a later
+     * AssignTrainingPoints on sampled data; here that map is left alone.
+     */
+    void PrepareQueries(const float* data_to_cluster, const vector_value_t* queries, const size_t n_queries,
+                        const bool on_device) {
+        centroids_to_explore = std::max<size_t>(static_cast<size_t>(n_clusters * config.ann_explore_fraction), 1);
+        if (config.verbose) {
+            std::cout << "Centroids to explore: " << centroids_to_explore << " ("
+                      << config.ann_explore_fraction * 100.0f << "% of " << n_clusters << ")" << std::endl;
+        }
+        if (config.objective_k == 0 || config.objective_k > 1024 || centroids_to_explore > 1024) {
+            throw std::invalid_argument(
+                "recall tracking supports objective_k and n_clusters * ann_explore_fraction up to 1024");
+        }
+        rotated_queries.Reset(ctx, n_queries * d);
+        if (config.sample_queries) {
+            if (n_queries > n_samples) {
+                throw std::invalid_argument("cannot sample more queries than there are training samples");
+            }
+            if (n_queries < n_samples) {
+                std::mt19937 rng(config.seed);
+                std::vector<size_t> order(n_samples);
+                std::iota(order.begin(), order.end(), size_t{0});
+                std::shuffle(order.begin(), order.end(), rng);
+                std::vector<uint64_t> rows(order.begin(), order.begin() + n_queries);
+                dbuf<uint64_t> d_rows(ctx, n_queries);
+                d_rows.Upload(rows.data(), n_queries);
+                hip::Check(skm_gather_rows(ctx, data_to_cluster, d, d_rows.get(), n_queries, rotated_queries.get(),
+                                           nullptr, nullptr));
+                hip::Check(skm_sync(ctx));
+            } else {
+                hip::Check(skm_copy(ctx, rotated_queries.get(), data_to_cluster, sizeof(float) * n_queries * d));
+            }
+        } else if (on_device) {
+            RotateOrCopy(queries, rotated_queries.get(), n_queries, !config.data_already_rotated);
+        } else {
+            dbuf<float> raw(ctx, n_queries * d);
+            raw.Upload(queries, n_queries * d);
+            RotateOrCopy(raw.get(), rotated_queries.get(), n_queries, !config.data_already_rotated);
+            hip::Check(skm_sync(ctx));  // `raw` is released on return
+        }
+        query_norms.Reset(ctx, n_queries);
+        gt_assignments.Reset(ctx, n_queries * config.objective_k);
+        gt_distances.Reset(ctx, n_queries * config.objective_k);
+        promising_centroids.Reset(ctx, n_queries * centroids_to_explore);
+        recall_distances.Reset(ctx, n_queries * centroids_to_explore);
+        hip::Check(skm_norms(ctx, rotated_queries.get(), n_queries, d, d, query_norms.get()));
+        hip::Check(skm_knn(ctx, rotated_queries.get(), n_queries, data_to_cluster, n_samples, d, query_norms.get(),
+                           data_norms.get(), config.objective_k, gt_assignments.get(), gt_distances.get()));
+        n_tracked_queries = n_queries;
+    }
+
+    /**
+     * recall@objective_k of the current centroids (reference superkmeans.h:1044-1087): the share of a query's
+     * ground-truth neighbours whose cluster is among the query's centroids_to_explore nearest centroids,
+     * averaged over the queries with the reference's fp32 accumulation order.  centroid_norms must hold the
+     * full norms of horizontal_centroids.
+     */
+    float ComputeRecall(const size_t n_samples_, const size_t k) {
+        const size_t nq = n_tracked_queries;
+        hip::Check(skm_knn(ctx, rotated_queries.get(), nq, horizontal_centroids.get(), k, d, query_norms.get(),
+                           centroid_norms.get(), centroids_to_explore, promising_centroids.get(),
+                           recall_distances.get()));
+        std::vector<uint32_t> hits(nq);
+        hip::Check(skm_recall_hits(ctx, gt_assignments.get(), promising_centroids.get(), d_assignments.get(),
+                                   n_samples_, nq, config.objective_k, centroids_to_explore, hits.data()));
+        float sum_recall = 0.0f;
+        for (size_t i = 0; i < nq; ++i) {
+            sum_recall += static_cast<float>(hits[i]) / static_cast<float>(config.objective_k);
+        }
+        return sum_recall / static_cast<float>(nq);
     }
 
     /**
@@ -726,6 +809,12 @@ class SuperKMeans {
     // Host state
     std::unique_ptr<uint32_t[]> cluster_sizes;
     std::unique_ptr<size_t[]> sampled_indices;
+
+    // Recall tracking (training with queries): device-resident lists.
+    size_t n_tracked_queries = 0;
+    size_t centroids_to_explore = 0;
+    dbuf<float> rotated_queries, query_norms, gt_distances, recall_distances;
+    dbuf<uint32_t> gt_assignments, promising_centroids;
     std::vector<float> host_distances;
     bool collect_prune_accounting = false;
     std::vector<std::vector<uint64_t>> prune_accounting;

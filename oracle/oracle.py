@@ -342,6 +342,14 @@ class KMeans:
         self._check(self.lib.oracle_kmeans_train(self.h, _fp(data), c_size_t(data.shape[0]), q, c_size_t(nq), _fp(out)))
         return out
 
+    def train_sampled_queries(self, data, n_queries):
+        """Train with n_queries queries drawn from the data (config sample_queries=1, no query pointer)."""
+        data = f32(data)
+        out = np.empty((self.k, self.d), dtype=np.float32)
+        self._check(self.lib.oracle_kmeans_train(self.h, _fp(data), c_size_t(data.shape[0]), None,
+                                                 c_size_t(n_queries), _fp(out)))
+        return out
+
     def assign(self, vectors, centroids):
         vectors, centroids = f32(vectors), f32(centroids)
         out = np.empty(vectors.shape[0], dtype=np.uint32)

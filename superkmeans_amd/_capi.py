@@ -69,7 +69,7 @@ _PROTOTYPES = {
     "skm_kmeans_create": (c_int, [c_size_t, c_size_t, c_void_p, c_int, POINTER(c_void_p)]),
     "skm_kmeans_destroy": (c_int, [c_void_p]),
     "skm_kmeans_train": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p, c_size_t, c_void_p]),
-    "skm_kmeans_train_device": (c_int, [c_void_p, _F, c_size_t, c_void_p]),
+    "skm_kmeans_train_device": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_void_p]),
     "skm_kmeans_assign": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
     "skm_kmeans_assign_device": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, _F]),
     "skm_kmeans_assign_training_points": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, c_void_p]),
@@ -314,16 +314,23 @@ class KMeans:
         except Exception:
             pass
 
-    def train(self, data):
+    def train(self, data, queries=None, n_queries=0):
+        """`queries`: (n_queries, d) array, or None with n_queries > 0 when the config samples them."""
         data = np.ascontiguousarray(data, dtype=np.float32)
         out = np.empty((self.k, self.d), dtype=np.float32)
-        check(self.lib.skm_kmeans_train(self.handle, data.ctypes.data, data.shape[0], None, 0, out.ctypes.data))
+        qptr = None
+        if queries is not None:
+            queries = np.ascontiguousarray(queries, dtype=np.float32)
+            qptr, n_queries = queries.ctypes.data, queries.shape[0]
+        check(self.lib.skm_kmeans_train(self.handle, data.ctypes.data, data.shape[0], qptr, n_queries,
+                                        out.ctypes.data))
         return out
 
-    def train_device(self, d_data, n):
+    def train_device(self, d_data, n, d_queries=None, n_queries=0):
         out = np.empty((self.k, self.d), dtype=np.float32)
         ptr = d_data.ptr if isinstance(d_data, DeviceArray) else d_data
-        check(self.lib.skm_kmeans_train_device(self.handle, ptr, n, out.ctypes.data))
+        qptr = d_queries.ptr if isinstance(d_queries, DeviceArray) else d_queries
+        check(self.lib.skm_kmeans_train_device(self.handle, ptr, n, qptr, n_queries, out.ctypes.data))
         return out
 
     def assign(self, vectors, centroids):

@@ -136,11 +136,13 @@ int skm_kmeans_train(skm_kmeans* km, const float* h_data, size_t n, const float*
     });
 }
 
-int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, float* h_out_centroids) {
+int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, const float* d_queries, size_t n_queries,
+                            float* h_out_centroids) {
     if (!km || !d_data || !h_out_centroids)
         return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_train_device: null argument");
     SKM_API_GUARD({
-        auto c = km->hier ? km->hier->TrainDevice(d_data, n) : km->flat->TrainDevice(d_data, n);
+        auto c = km->hier ? km->hier->TrainDevice(d_data, n, d_queries, n_queries)
+                          : km->flat->TrainDevice(d_data, n, d_queries, n_queries);
         std::memcpy(h_out_centroids, c.data(), c.size() * sizeof(float));
         km->n_trained = n;
     });

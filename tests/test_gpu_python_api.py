@@ -115,3 +115,17 @@ def test_assign_training_points_agrees_with_assign(pkg, blobs):
 
     with pytest.raises(RuntimeError, match="trained first"):  # superkmeans.h:404-406
         _superkmeans.SuperKMeans(k, d).assign_training_points(data, c)
+
+
+def test_train_with_queries(pkg):  # python/tests/test_superkmeans.py:49-64 of the reference
+    np.random.seed(42)
+    n, d, k, q = 10000, 512, 100, 50
+    data = np.random.randn(n, d).astype(np.float32)
+    queries = np.random.randn(q, d).astype(np.float32)
+    km = pkg.SuperKMeans(n_clusters=k, dimensionality=d, iters=5, objective_k=10, verbose=False)
+    centroids = km.train(data, queries=queries)
+    assert centroids.shape == (k, d) and km.is_trained_ and len(km.iteration_stats) > 0
+    assert all(0.0 <= s.recall <= 1.0 for s in km.iteration_stats)
+    assert any(s.recall > 0.0 for s in km.iteration_stats)
+    with pytest.raises(ValueError, match="dimensionality"):
+        pkg.SuperKMeans(n_clusters=k, dimensionality=d).train(data, queries=queries[:, :100].copy())

@@ -237,3 +237,71 @@ def test_hierarchical_train_matches_oracle(capi, ctx, oracle, blobs, n, d, k):
     used = len(np.unique(km.assign(X, C)))
     assert used >= 0.95 * k  # test_hierarchical_superkmeans.cpp:554-587
     km.close()
+
+
+@pytest.mark.parametrize("mode", ["given", "sampled", "device"])
+def test_flat_train_with_queries_tracks_recall_like_oracle(capi, ctx, oracle, blobs, mode):
+    """Training with queries (superkmeans.h:243-274, 848-851): same recall per iteration as the oracle.
+    Recall is a mean of integer hit counts over n_q * objective_k pairs; one near-tie resolved differently
+    moves it by 1 / (n_q * objective_k), so the bar is a handful of such quanta."""
+    n, d, k, nq, ok_, iters = 12000, 128, 200, 64, 10, 6
+    X = blobs(n, d, k, std=0.35, seed=21)
+    Q = blobs(nq, d, k, std=0.35, seed=22)
+    cfg = dict(iters=iters, sampling_fraction=1.0, early_termination=0, objective_k=ok_, ann_explore_fraction=0.05,
+               sample_queries=1 if mode == "sampled" else 0)
+    km, okm = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    if mode == "given":
+        C = km.train(X, queries=Q)
+        OC = okm.train(X, queries=Q)
+    elif mode == "device":
+        dX, dQ = km.ctx.array(X), km.ctx.array(Q)
+        C = km.train_device(dX, n, dQ, nq)
+        OC = okm.train(X, queries=Q)
+        dX.free(), dQ.free()
+    else:
+        C = km.train(X, n_queries=nq)
+        OC = okm.train_sampled_queries(X, nq)
+    gs, os_ = km.stats(), okm.stats()
+    assert len(gs) == len(os_) == iters
+    quantum = 1.0 / (nq * ok_)
+    for a, b in zip(gs, os_):
+        assert 0.0 <= a.recall <= 1.0
+        assert abs(a.recall - b.recall) <= 5 * quantum + 1e-6, (a.iteration, a.recall, b.recall)
+        assert abs(a.objective - b.objective_f64) <= 1e-3 * b.objective_f64
+    assert gs[0].recall == pytest.approx(os_[0].recall, abs=1e-7)  # first iteration: no split-induced ties yet
+    assert gs[-1].recall >= gs[0].recall - 0.05  # clustering does not get worse for the queries
+    assert _rel_l2(C, OC) <= 1e-2
+    km.close()
+
+
+def test_flat_train_recall_early_termination_matches_oracle(capi, ctx, oracle, blobs):
+    # well-separated blobs: recall saturates at once, so the patience rule (superkmeans.h:1315-1331) stops
+    # the run after RECALL_CONVERGENCE_PATIENCE iterations without improvement unless tol/shift stop it first
+    n, d, k, nq = 8000, 128, 150, 50
+    X = blobs(n, d, k, std=0.05, seed=31)
+    Q = blobs(nq, d, k, std=0.05, seed=32)
+    cfg = dict(iters=30, sampling_fraction=1.0, early_termination=1, objective_k=10, ann_explore_fraction=0.1, tol=0.0)
+    km, okm = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    km.train(X, queries=Q)
+    okm.train(X, queries=Q)
+    assert len(km.stats()) == len(okm.stats()) < 30
+    assert [round(s.recall, 4) for s in km.stats()] == [round(s.recall, 4) for s in okm.stats()]
+    km.close()
+
+
+def test_train_with_queries_argument_errors(capi, ctx, blobs):
+    X = blobs(3000, 64, 20, std=0.3, seed=1)
+    km = capi.KMeans(20, 64, iters=2, sampling_fraction=1.0)
+    with pytest.raises(capi.SkmError, match="Queries must be provided"):
+        km.train(X, n_queries=10)  # no pointer and sample_queries is off (superkmeans.h:178-182)
+    km.close()
+    km = capi.KMeans(20, 64, iters=2, sampling_fraction=1.0, objective_k=5000)
+    with pytest.raises(capi.SkmError, match="1024"):
+        km.train(X, queries=X[:10])
+    km.close()
+    # the hierarchical driver ignores queries (hierarchical_superkmeans.h:77,94-99)
+    hk = capi.KMeans(20, 64, hierarchical=True, iters_mesoclustering=2, iters_fineclustering=2, iters_refinement=1,
+                     sampling_fraction=1.0, suppress_warnings=1)
+    C = hk.train(X, queries=X[:10])
+    assert C.shape == (20, 64) and all(s.recall == 0.0 for s in hk.stats(3))
+    hk.close()
