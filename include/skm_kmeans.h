@@ -48,6 +48,10 @@ typedef struct skm_kmeans_config {
     uint32_t iters_mesoclustering;
     uint32_t iters_fineclustering;
     uint32_t iters_refinement;
+    /* Rotation variant; a build option of the reference (pdx/adsampling.h:52-74), a field here:
+     * 0 dense Gaussian matrix, 1 sign flip + DCT-II when d >= 512 and d is a power of two, 2 DCT
+     * whenever d >= 512. */
+    int32_t dct_rotation;
 } skm_kmeans_config;
 
 /* SuperKMeansIterationStats (superkmeans.h:60-72). */
@@ -109,9 +113,11 @@ int skm_kmeans_get_prune_accounting(skm_kmeans* km, size_t iteration, uint64_t* 
                                     size_t* out_len, size_t* out_rows);
 /* PDXLayout::GetDimensionSplit (pdx/layout.h:115-140) as used by the host code. */
 void skm_dimension_split(size_t d, size_t* out_horizontal_d, size_t* out_vertical_d);
-/* ADSamplingPruner matrix and ratios as built by the host code for (d, epsilon0, seed): fills
+/* ADSamplingPruner matrix and ratios as built by the host code for (d, epsilon0, seed) and the
+ * rotation variant `rotation_kind` (the values of skm_kmeans_config.dct_rotation): fills
  * h_out_matrix (d*d, may be NULL) and h_out_ratios (d+1, may be NULL). Needs a device. */
-int skm_pruner_tables(size_t d, float epsilon0, uint32_t seed, float* h_out_matrix, float* h_out_ratios);
+int skm_pruner_tables(size_t d, float epsilon0, uint32_t seed, int rotation_kind, float* h_out_matrix,
+                      float* h_out_ratios);
 
 #ifdef __cplusplus
 }

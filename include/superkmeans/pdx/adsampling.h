@@ -1,8 +1,10 @@
 // ADSampling pruner, HIP backend: threshold ratios and the random orthogonal rotation.
 //
-// Mirrors the interface of the reference's ADSamplingPruner (pdx/adsampling.h:29-328, dense-matrix
-// variant): the ratios table, Rotate and Unrotate.  The d x d matrix is built on the host and kept
-// on the device (Q and Q^T); Rotate/Unrotate are MFMA GEMMs (skm_rotate / skm_unrotate).
+// Mirrors the interface of the reference's ADSamplingPruner (pdx/adsampling.h:29-328): the ratios
+// table, Rotate and Unrotate.  The d x d matrix is built on the host and kept on the device (Q and
+// Q^T); Rotate/Unrotate are MFMA GEMMs (skm_rotate / skm_unrotate).  Both rotations of the reference
+// are orthonormal matrices, so both run through the same GEMM: the dense Gaussian one (default build
+// of the reference) and the sign flip + DCT-II one (reference builds with FFTW, d >= 512).
 #pragma once
 
 #include <cmath>
@@ -72,6 +74,43 @@ inline std::vector<float> OrthogonalFactor(std::vector<double> a, const size_t d
     return out;
 }
 
+// Which rotation the pruner builds (reference pdx/adsampling.h:52-85).
+enum RotationKind : int {
+    kRotationDense = 0,        // Q of a Gaussian matrix: reference builds without FFTW
+    kRotationDctPow2Only = 1,  // DCT when d >= 512 and d is a power of two: FFTW builds with AVX2
+    kRotationDct = 2           // DCT when d >= 512: FFTW builds without AVX2
+};
+
+inline bool UsesDctRotation(const int kind, const size_t d) {
+    if (kind == kRotationDense || d < D_THRESHOLD_FOR_DCT_ROTATION) return false;
+    if (kind == kRotationDctPow2Only) return (d & (d - 1)) == 0;
+    return true;
+}
+
+// Sign flip followed by the orthonormal DCT-II, as one matrix (pdx/adsampling.h:60-71,162-189):
+// Q[k][j] = sign_j * c_k * cos(pi * (j + 1/2) * k / d), c_0 = sqrt(1/d), c_k = sqrt(2/d);
+// sign_j = +1 where std::uniform_int_distribution<int>(0, 1) over std::mt19937(seed) draws 1.
+// FFTW's REDFT10 returns 2 * sum_j x_j cos(...); the reference scales bin 0 by sqrt(1/(4d)) and the
+// others by sqrt(1/(2d)), which gives the c_k above.
+inline std::vector<float> DctRotationMatrix(const size_t d, const uint32_t seed) {
+    std::mt19937 gen(seed);
+    std::uniform_int_distribution<int> dist(0, 1);
+    std::vector<double> sign(d);
+    for (size_t j = 0; j < d; ++j) sign[j] = dist(gen) ? 1.0 : -1.0;
+    const double pi = 3.14159265358979323846;
+    const double c0 = std::sqrt(1.0 / static_cast<double>(d)), c = std::sqrt(2.0 / static_cast<double>(d));
+    std::vector<float> out(d * d);
+    for (size_t k = 0; k < d; ++k) {
+        for (size_t j = 0; j < d; ++j) {
+            // (2j + 1) * k reduced modulo 4d keeps the cosine argument small and exact for large d
+            const size_t m = ((2 * j + 1) * k) % (4 * d);
+            const double v = std::cos(pi * static_cast<double>(m) / (2.0 * static_cast<double>(d)));
+            out[k * d + j] = static_cast<float>(sign[j] * (k == 0 ? c0 : c) * v);
+        }
+    }
+    return out;
+}
+
 } // namespace detail
 
 template <Quantization q = Quantization::f32>
@@ -83,15 +122,21 @@ class ADSamplingPruner {
     // Draws d*d N(0,1) values row by row from std::mt19937(seed) through
     // std::normal_distribution<float> (the reference's sequence, pdx/adsampling.h:76-82) and keeps
     // the orthogonal factor of their QR decomposition.
-    ADSamplingPruner(skm_ctx* ctx, uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42)
+    // With a DCT rotation kind that applies to this d, the matrix is the sign flip + DCT-II instead.
+    ADSamplingPruner(skm_ctx* ctx, uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42,
+                     int rotation_kind = detail::kRotationDense)
         : num_dimensions(num_dimensions_), ctx_(ctx), epsilon0(epsilon0_) {
         InitializeRatios();
         const size_t d = num_dimensions;
-        std::mt19937 gen(seed);
-        std::normal_distribution<float> dist(0.0f, 1.0f);
-        std::vector<double> a(d * d);
-        for (size_t i = 0; i < d * d; ++i) a[i] = dist(gen);
-        matrix_ = detail::OrthogonalFactor(std::move(a), d);
+        if (detail::UsesDctRotation(rotation_kind, d)) {
+            matrix_ = detail::DctRotationMatrix(d, seed);
+        } else {
+            std::mt19937 gen(seed);
+            std::normal_distribution<float> dist(0.0f, 1.0f);
+            std::vector<double> a(d * d);
+            for (size_t i = 0; i < d * d; ++i) a[i] = dist(gen);
+            matrix_ = detail::OrthogonalFactor(std::move(a), d);
+        }
         d_q_.Reset(ctx_, d * d);
         d_qt_.Reset(ctx_, d * d);
         d_q_.Upload(matrix_.data(), d * d);

@@ -58,6 +58,11 @@ struct SuperKMeansConfig {
     bool suppress_warnings = false;
 
     bool data_already_rotated = false;
+
+    // Not in the reference's struct, where it is a build option (FFTW present or not): which rotation the
+    // pruner uses.  0 = dense Gaussian (builds without FFTW), 1 = sign flip + DCT-II when d >= 512 and d
+    // is a power of two (FFTW builds on AVX2 machines), 2 = DCT whenever d >= 512 (other FFTW builds).
+    int dct_rotation = 0;
 };
 
 struct SuperKMeansIterationStats {
@@ -123,7 +128,8 @@ class SuperKMeans {
         g_n_threads = n_threads;
         context = std::make_shared<hip::Context>(0);
         ctx = context->get();
-        pruner = std::make_unique<pruner_t>(ctx, dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed);
+        pruner = std::make_unique<pruner_t>(ctx, dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed,
+                                            config.dct_rotation);
         if (this->config.data_already_rotated) {
             this->config.unrotate_centroids = false;
         }

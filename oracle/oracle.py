@@ -42,6 +42,7 @@ class Config(ctypes.Structure):
         ("iters_mesoclustering", c_uint32),
         ("iters_fineclustering", c_uint32),
         ("iters_refinement", c_uint32),
+        ("dct_rotation", ctypes.c_int32),
     ]
 
 
@@ -189,6 +190,18 @@ def find_nn(x, y, norms_x=None, norms_y=None):
     load().oracle_find_nn(_fp(x), _fp(y), c_size_t(x.shape[0]), c_size_t(y.shape[0]), c_size_t(x.shape[1]), _fp(nx),
                           _fp(ny), _fp(knn), _fp(dist))
     return knn, dist
+
+
+def rotate_kind(x, seed=42, rotation_kind=1, forward=True, want_matrix=False):
+    """Rotate / Unrotate of the pruner built for `rotation_kind` (1, 2: DCT variants of pdx/adsampling.h:52-74).
+    Returns (out, uses_dct[, matrix])."""
+    x = f32(x)
+    n, d = x.shape
+    out = np.empty_like(x)
+    m = np.empty((d, d), dtype=np.float32) if want_matrix else None
+    used = load().oracle_rotate_kind(c_uint32(d), c_uint32(seed), c_int(rotation_kind), c_int(1 if forward else 0),
+                                     _fp(x), c_uint32(n), _fp(out), _fp(m) if want_matrix else None)
+    return (out, bool(used), m) if want_matrix else (out, bool(used))
 
 
 def find_knn(x, y, k, norms_x=None, norms_y=None):

@@ -175,7 +175,12 @@ static inline float Horizontal(const float* v1, const float* v2, size_t num_dime
     return distance;
 }
 
-// ---- pdx/adsampling.h: pruner (dense-matrix variant; the FFTW/DCT branch is not built) ----
+// ---- pdx/adsampling.h: pruner.  Dense-matrix variant and, on request, the FFTW/DCT variant ----
+// FFTW is not available, so the DCT branch (adsampling.h:60-71,162-189,229-271) is restated from the
+// definitions of the transforms FFTW documents: REDFT10 Y_k = 2 sum_j X_j cos(pi (j + 1/2) k / n) and
+// REDFT01 Y_k = X_0 + 2 sum_{j>=1} X_j cos(pi j (k + 1/2) / n), evaluated directly in double (O(d^2) per
+// vector), with the reference's sign flip and scale factors around them.  PARITY UNPINNED at the level of
+// FFTW's fp32 butterflies; pinned against scipy.fft.dct(norm="ortho") in the tests.
 // The rotation matrix is the Q factor of a Householder QR of a d x d matrix of N(0,1) draws
 // (adsampling.h:76-85).  Eigen is unavailable, so the factorisation is a textbook Householder QR in
 // double precision; the value sequence of the draws (std::mt19937 + std::normal_distribution<float>,
@@ -190,10 +195,80 @@ class ADSamplingPruner {
     std::vector<float> ratios;
     std::vector<float> matrix;  // d x d row-major
 
-    ADSamplingPruner(uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42)
+    bool use_dct = false;
+    std::vector<float> flip;      // +1 / -1 per dimension (adsampling.h:60-70)
+    std::vector<double> cos_tab;  // cos(pi (j + 1/2) k / d) at [k * d + j]
+
+    // rotation_kind: 0 dense, 1 DCT when d >= 512 and a power of two (HAS_FFTW && __AVX2__), 2 DCT when
+    // d >= 512 (HAS_FFTW otherwise); adsampling.h:52-59.
+    ADSamplingPruner(uint32_t num_dimensions_, float epsilon0_, uint32_t seed = 42, int rotation_kind = 0)
         : num_dimensions(num_dimensions_), epsilon0(epsilon0_) {
         InitializeRatios();
-        MakeRotationMatrix(num_dimensions, seed, matrix);
+        const size_t d = num_dimensions;
+        const bool pow2 = (d & (d - 1)) == 0;
+        use_dct = rotation_kind != 0 && d >= 512 && (rotation_kind == 2 || pow2);
+        if (!use_dct) {
+            MakeRotationMatrix(num_dimensions, seed, matrix);
+            return;
+        }
+        std::mt19937 gen(seed);
+        std::uniform_int_distribution<int> dist(0, 1);
+        flip.resize(d);
+        for (size_t i = 0; i < d; ++i) flip[i] = dist(gen) ? 1.0f : -1.0f;
+        cos_tab.resize(d * d);
+        const double pi = 3.14159265358979323846;
+        for (size_t k = 0; k < d; ++k)
+            for (size_t j = 0; j < d; ++j)
+                cos_tab[k * d + j] = std::cos(pi * (static_cast<double>(j) + 0.5) * static_cast<double>(k) /
+                                              static_cast<double>(d));
+        // The explicit matrix, for callers that ask for it: row k = image of nothing, column j = R e_j.
+        matrix.resize(d * d);
+        std::vector<float> e(d, 0.0f), col(d);
+        for (size_t j = 0; j < d; ++j) {
+            e[j] = 1.0f;
+            RotateDct(e.data(), col.data(), 1);
+            e[j] = 0.0f;
+            for (size_t k = 0; k < d; ++k) matrix[k * d + j] = col[k];
+        }
+    }
+
+    // adsampling.h:162-189: FlipSign, REDFT10 in place, column 0 scaled by sqrt(1/(4d)), the rest by sqrt(1/(2d)).
+    void RotateDct(const float* vectors, float* out_buffer, const uint32_t n) const {
+        const size_t d = num_dimensions;
+        const float s0 = std::sqrt(1.0f / (4.0f * num_dimensions));
+        const float s = std::sqrt(1.0f / (2.0f * num_dimensions));
+#pragma omp parallel for num_threads(g_n_threads)
+        for (size_t i = 0; i < (size_t) n; ++i) {
+            std::vector<float> x(d);
+            for (size_t j = 0; j < d; ++j) x[j] = vectors[i * d + j] * flip[j];
+            for (size_t k = 0; k < d; ++k) {
+                double acc = 0.0;
+                const double* c = &cos_tab[k * d];
+                for (size_t j = 0; j < d; ++j) acc += static_cast<double>(x[j]) * c[j];
+                const float y = static_cast<float>(2.0 * acc);
+                out_buffer[i * d + k] = y * (k == 0 ? s0 : s);
+            }
+        }
+    }
+
+    // adsampling.h:229-271: undo the scaling, REDFT01, times 1/(2d), FlipSign.
+    void UnrotateDct(const float* rotated, float* out_buffer, const uint32_t n) const {
+        const size_t d = num_dimensions;
+        const float inv_s0 = std::sqrt(4.0f * num_dimensions);
+        const float inv_s = std::sqrt(2.0f * num_dimensions);
+        const float norm = 1.0f / (2.0f * num_dimensions);
+#pragma omp parallel for num_threads(g_n_threads)
+        for (size_t i = 0; i < (size_t) n; ++i) {
+            std::vector<float> x(d);
+            for (size_t j = 0; j < d; ++j) x[j] = rotated[i * d + j] * (j == 0 ? inv_s0 : inv_s);
+            for (size_t k = 0; k < d; ++k) {
+                double acc = 0.0;
+                // cos(pi j (k + 1/2) / d) is the transposed entry of the forward table
+                for (size_t j = 1; j < d; ++j) acc += static_cast<double>(x[j]) * cos_tab[j * d + k];
+                const float y = static_cast<float>(static_cast<double>(x[0]) + 2.0 * acc);
+                out_buffer[i * d + k] = (y * norm) * flip[k];
+            }
+        }
     }
 
     // adsampling.h:93-99
@@ -204,11 +279,13 @@ class ADSamplingPruner {
 
     // adsampling.h:156-216 (dense branch): out = vectors * matrix^T
     void Rotate(const float* vectors, float* out_buffer, const uint32_t n) const {
+        if (use_dct) return RotateDct(vectors, out_buffer, n);
         sgemm('T', 'N', (int) num_dimensions, (int) n, (int) num_dimensions, matrix.data(), (int) num_dimensions,
               vectors, (int) num_dimensions, out_buffer, (int) num_dimensions);
     }
     // adsampling.h:223-299 (dense branch): out = rotated * matrix
     void Unrotate(const float* rotated, float* out_buffer, const uint32_t n) const {
+        if (use_dct) return UnrotateDct(rotated, out_buffer, n);
         sgemm('N', 'N', (int) num_dimensions, (int) n, (int) num_dimensions, matrix.data(), (int) num_dimensions,
               rotated, (int) num_dimensions, out_buffer, (int) num_dimensions);
     }
@@ -600,6 +677,7 @@ struct Config {  // superkmeans.h:23-55 + hierarchical_superkmeans.h:11-17, C la
     uint32_t iters_mesoclustering;
     uint32_t iters_fineclustering;
     uint32_t iters_refinement;
+    int32_t dct_rotation;  // 0: build without FFTW; 1: HAS_FFTW && __AVX2__; 2: HAS_FFTW (adsampling.h:52-59)
 };
 
 struct IterationStats {  // superkmeans.h:60-72
@@ -633,13 +711,15 @@ class KMeans {
         g_n_threads = n_threads;
         if (hierarchical) {
             // hierarchical_superkmeans.h:48-65
-            pruner = std::make_unique<ADSamplingPruner>(dimensionality, HIERARCHICAL_PRUNER_INITIAL_THRESHOLD, config.seed);
+            pruner = std::make_unique<ADSamplingPruner>(dimensionality, HIERARCHICAL_PRUNER_INITIAL_THRESHOLD, config.seed,
+                                                        config.dct_rotation);
             ENSURE_POSITIVE(config.iters_mesoclustering);
             ENSURE_POSITIVE(config.iters_fineclustering);
             if (n_clusters <= 128 && !config.suppress_warnings)
                 printf("WARNING: n_clusters <= 128 is not recommended for HierarchicalSuperKMeans. Consider using at least 128 clusters.\n");
         } else {
-            pruner = std::make_unique<ADSamplingPruner>(dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed);
+            pruner = std::make_unique<ADSamplingPruner>(dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed,
+                                                        config.dct_rotation);
         }
         if (config.data_already_rotated) config.unrotate_centroids = false;
     }
@@ -854,6 +934,7 @@ class KMeans {
         c.iters_mesoclustering = 3;
         c.iters_fineclustering = 5;
         c.iters_refinement = 0;
+        c.dct_rotation = 0;
         return c;
     }
 
@@ -1553,6 +1634,18 @@ void oracle_ratios(uint32_t d, float epsilon0, float* out) {
 void oracle_rotation_matrix(uint32_t d, uint32_t seed, float* out) {
     ADSamplingPruner p(d, PRUNER_INITIAL_THRESHOLD, seed);
     std::memcpy(out, p.matrix.data(), sizeof(float) * (size_t) d * d);
+}
+// Rotation of the DCT variant (rotation_kind 1 or 2); forward != 0: Rotate, else Unrotate.  out_matrix (d*d, may
+// be NULL) receives the equivalent explicit matrix.  Returns 1 when the variant applies to this d, else 0
+// (then the dense rotation is used, as in the reference).
+int oracle_rotate_kind(uint32_t d, uint32_t seed, int rotation_kind, int forward, const float* x, uint32_t n,
+                       float* out, float* out_matrix) {
+    ADSamplingPruner p(d, 1.5f, seed, rotation_kind);
+    if (x && out) {
+        if (forward) p.Rotate(x, out, n); else p.Unrotate(x, out, n);
+    }
+    if (out_matrix) std::memcpy(out_matrix, p.matrix.data(), sizeof(float) * d * d);
+    return p.use_dct ? 1 : 0;
 }
 void oracle_rotate(const float* q, uint32_t d, const float* x, uint32_t n, float* out) {
     sgemm('T', 'N', (int) d, (int) n, (int) d, q, (int) d, x, (int) d, out, (int) d);

@@ -83,7 +83,7 @@ _PROTOTYPES = {
     "skm_kmeans_get_prune_accounting": (
         c_int, [c_void_p, c_size_t, c_void_p, c_size_t, POINTER(c_size_t), POINTER(c_size_t)]),
     "skm_dimension_split": (None, [c_size_t, POINTER(c_size_t), POINTER(c_size_t)]),
-    "skm_pruner_tables": (c_int, [c_size_t, c_float, c_uint32, c_void_p, c_void_p]),
+    "skm_pruner_tables": (c_int, [c_size_t, c_float, c_uint32, c_int, c_void_p, c_void_p]),
 }
 
 
@@ -114,6 +114,7 @@ class KMeansConfig(ctypes.Structure):
         ("iters_mesoclustering", c_uint32),
         ("iters_fineclustering", c_uint32),
         ("iters_refinement", c_uint32),
+        ("dct_rotation", c_int),
     ]
 
 
@@ -393,10 +394,10 @@ def dimension_split(d):
     return h.value, v.value
 
 
-def pruner_tables(d, epsilon0=1.5, seed=42):
+def pruner_tables(d, epsilon0=1.5, seed=42, rotation_kind=0):
     m = np.empty((d, d), dtype=np.float32)
     r = np.empty(d + 1, dtype=np.float32)
-    check(load().skm_pruner_tables(d, epsilon0, seed, m.ctypes.data, r.ctypes.data))
+    check(load().skm_pruner_tables(d, epsilon0, seed, rotation_kind, m.ctypes.data, r.ctypes.data))
     return m, r
 
 

@@ -118,6 +118,7 @@ PYBIND11_MODULE(_superkmeans, m) {
         .def_readwrite("objective_k", &SuperKMeansConfig::objective_k)
         .def_readwrite("verbose", &SuperKMeansConfig::verbose)
         .def_readwrite("angular", &SuperKMeansConfig::angular)
+        .def_readwrite("dct_rotation", &SuperKMeansConfig::dct_rotation)
         .def("__repr__", [](const SuperKMeansConfig& c) {
             return "<SuperKMeansConfig: iters=" + std::to_string(c.iters) +
                    ", sampling_fraction=" + std::to_string(c.sampling_fraction) +

@@ -41,6 +41,7 @@ void fill_base(skmeans::SuperKMeansConfig& c, const skm_kmeans_config& in) {
     c.angular = in.angular != 0;
     c.suppress_warnings = in.suppress_warnings != 0;
     c.data_already_rotated = in.data_already_rotated != 0;
+    c.dct_rotation = in.dct_rotation;
 }
 
 } // namespace
@@ -95,6 +96,7 @@ void skm_kmeans_default_config(skm_kmeans_config* out, int hierarchical) {
     out->iters_mesoclustering = h.iters_mesoclustering;
     out->iters_fineclustering = h.iters_fineclustering;
     out->iters_refinement = h.iters_refinement;
+    out->dct_rotation = c.dct_rotation;
 }
 
 int skm_kmeans_create(size_t n_clusters, size_t dimensionality, const skm_kmeans_config* config, int hierarchical,
@@ -262,11 +264,12 @@ void skm_dimension_split(size_t d, size_t* out_horizontal_d, size_t* out_vertica
     if (out_vertical_d) *out_vertical_d = s.vertical_d;
 }
 
-int skm_pruner_tables(size_t d, float epsilon0, uint32_t seed, float* h_out_matrix, float* h_out_ratios) {
+int skm_pruner_tables(size_t d, float epsilon0, uint32_t seed, int rotation_kind, float* h_out_matrix,
+                      float* h_out_ratios) {
     if (d == 0) return skm::set_error(SKM_ERR_INVALID, "skm_pruner_tables: d must be positive");
     SKM_API_GUARD({
         skmeans::hip::Context c(0);
-        skmeans::ADSamplingPruner<> p(c.get(), (uint32_t) d, epsilon0, seed);
+        skmeans::ADSamplingPruner<> p(c.get(), (uint32_t) d, epsilon0, seed, rotation_kind);
         if (h_out_matrix) std::memcpy(h_out_matrix, p.HostMatrix().data(), d * d * sizeof(float));
         if (h_out_ratios) std::memcpy(h_out_ratios, p.ratios.data(), (d + 1) * sizeof(float));
     });

@@ -305,3 +305,51 @@ def test_train_with_queries_argument_errors(capi, ctx, blobs):
     C = hk.train(X, queries=X[:10])
     assert C.shape == (20, 64) and all(s.recall == 0.0 for s in hk.stats(3))
     hk.close()
+
+
+def test_dct_rotation_variant_matches_oracle_and_scipy(capi, ctx, oracle, blobs):
+    """Rotation of reference builds with FFTW (pdx/adsampling.h:52-74,162-189): sign flip + orthonormal DCT-II,
+    here as an explicit matrix through the same GEMM."""
+    from scipy.fft import dct
+    d, seed = 512, 42
+    m, _ = capi.pruner_tables(d, 1.5, seed, rotation_kind=1)
+    x = np.random.default_rng(3).standard_normal((300, d)).astype(np.float32)
+    ref_out, used, om = oracle.rotate_kind(x, seed=seed, rotation_kind=1, want_matrix=True)
+    assert used and np.abs(m - om).max() <= 2e-7  # entries are at most sqrt(2/d) = 0.0625
+    dx, dq, dout = ctx.array(x), ctx.array(m), ctx.empty((300, d))
+    capi.check(ctx.lib.skm_rotate(ctx.handle, dx.ptr, 300, d, dq.ptr, dout.ptr))
+    got = dout.download()
+    draws = np.random.RandomState(seed).randint(0, 2 ** 32, size=d, dtype=np.uint64)
+    sign = np.where(draws >> 31 == 1, 1.0, -1.0)
+    exact = dct(x.astype(np.float64) * sign, type=2, norm="ortho", axis=1)
+    assert np.abs(got - exact).max() <= 1e-5 and np.abs(got - ref_out).max() <= 1e-5
+    for a in (dx, dq, dout):
+        a.free()
+    # d = 768 is not a power of two: kind 1 falls back to the dense matrix, kind 2 does not
+    dense, _ = capi.pruner_tables(768, 1.5, seed, rotation_kind=0)
+    assert np.array_equal(capi.pruner_tables(768, 1.5, seed, rotation_kind=1)[0], dense)
+    assert not np.array_equal(capi.pruner_tables(768, 1.5, seed, rotation_kind=2)[0], dense)
+    # whole Train under the DCT rotation, against the oracle's restatement of that branch
+    n, k = 12000, 300  # k > 256: iterations after the first one prune
+    X = blobs(n, d, k, std=0.3, seed=5)
+    cfg = dict(iters=5, sampling_fraction=1.0, early_termination=0, dct_rotation=1)
+    km, okm = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    C, OC = km.train(X), okm.train(X)
+    gs, os_ = km.stats(), okm.stats()
+    assert gs[0].is_gemm_only and not gs[1].is_gemm_only
+    for a, b in zip(gs, os_):
+        assert bool(a.is_gemm_only) == bool(b.is_gemm_only) and a.partial_d == b.partial_d and a.split == b.split
+        # after the first split the trajectories of two fp32 implementations separate (see
+        # test_flat_train_matches_oracle); the strict bar holds for the iterations before it
+        assert abs(a.objective - b.objective_f64) <= 1e-2 * b.objective_f64
+    for a, b in zip(gs[:2], os_[:2]):
+        assert abs(a.objective - b.objective_f64) <= 1e-4 * b.objective_f64
+        if not a.is_gemm_only:
+            assert abs(a.not_pruned_pct - b.not_pruned_pct) <= 1e-2 * max(b.not_pruned_pct, 1e-6) + 1e-6
+    assert abs(gs[-1].objective - os_[-1].objective_f64) <= 2e-3 * os_[-1].objective_f64
+    assert _rel_l2(C, OC) <= 2e-2
+    # centroids come back in the original space: their exact WCSS there equals the reported objective
+    a1 = km.assign(X, C)
+    wcss = ((X.astype(np.float64) - C.astype(np.float64)[a1]) ** 2).sum()
+    assert wcss <= km.stats()[-1].objective * (1 + 1e-3)
+    km.close()

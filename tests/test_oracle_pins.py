@@ -429,3 +429,34 @@ def test_recall_from_lists_by_hand(oracle):
     gt = np.array([[0, 1, 2, 3], [4, 5, 0, 1]], dtype=np.uint32)          # clusters [0,1,2,2] and [3,1,0,1]
     promising = np.array([[2, 7], [1, 3]], dtype=np.uint32)                # hits: 2 of 4, 3 of 4
     assert oracle.recall_from_lists(gt, promising, assign) == np.float32((np.float32(0.5) + np.float32(0.75)) / 2)
+
+
+# ---- DCT rotation variant (pdx/adsampling.h:52-74,162-189,229-271; reference builds with FFTW) ----
+def test_dct_rotation_equals_sign_flip_plus_orthonormal_dct(oracle):
+    from scipy.fft import dct
+    d, seed = 512, 42
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((50, d)).astype(np.float32)
+    out, used, m = oracle.rotate_kind(x, seed=seed, rotation_kind=1, want_matrix=True)
+    assert used
+    # signs: +1 where uniform_int_distribution<int>(0, 1) over mt19937(seed) draws 1, i.e. where the top bit
+    # of the 32-bit draw is set; numpy's RandomState seeds MT19937 the same way as std::mt19937(seed)
+    draws = np.random.RandomState(seed).randint(0, 2 ** 32, size=d, dtype=np.uint64)
+    sign = np.where(draws >> 31 == 1, 1.0, -1.0)
+    ref = dct(x.astype(np.float64) * sign, type=2, norm="ortho", axis=1)
+    assert np.abs(out - ref).max() <= 2e-6 * np.abs(ref).max()
+    m64 = m.astype(np.float64)
+    assert np.abs(m64 @ m64.T - np.eye(d)).max() <= 1e-5          # orthonormal
+    assert np.abs(x.astype(np.float64) @ m64.T - ref).max() <= 1e-5  # the explicit matrix is the same map
+    back, _ = oracle.rotate_kind(out, seed=seed, rotation_kind=1, forward=False)
+    assert np.abs(back - x).max() <= 1e-5                          # Unrotate inverts Rotate
+    assert np.allclose((out.astype(np.float64) ** 2).sum(1), (x.astype(np.float64) ** 2).sum(1), rtol=1e-5)
+
+
+def test_dct_rotation_applies_only_where_the_reference_would_use_it(oracle):
+    x = np.ones((1, 256), dtype=np.float32)
+    assert not oracle.rotate_kind(x, rotation_kind=1)[1] and not oracle.rotate_kind(x, rotation_kind=2)[1]  # d < 512
+    x = np.ones((1, 768), dtype=np.float32)
+    assert not oracle.rotate_kind(x, rotation_kind=1)[1]  # AVX2 builds: power of two only
+    assert oracle.rotate_kind(x, rotation_kind=2)[1]
+    assert not oracle.rotate_kind(np.ones((1, 1024), dtype=np.float32), rotation_kind=0)[1]
