@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace skm {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -141,9 +143,31 @@ __device__ __forceinline__ void mfma_step_tail(const float* as, const float* bs,
     }
 }
 
+// The 16 MFMAs of one group of 8 columns (fragments a0, a1, b0, b1 hold 4 columns each per lane).
+__device__ __forceinline__ void mfma_group(const floatx4& a0, const floatx4& a1, const floatx4& b0, const floatx4& b1,
+                                           WaveAcc& acc) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
+        acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
+        acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
+        acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
+    }
+}
+
 // Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are 16-byte aligned so operand
 // slices can be fetched with dwordx4 loads; then every full BK step is fetched without any guard (the
 // eight loads of a thread are issued back to back) and only a trailing partial step is guarded.
+//
+// Schedule of one full step kt (LDS buffer kt & 1 holds slice kt, registers hold slice kt + 1):
+//   1. slice kt + 1 goes from registers to the other LDS buffer (its last readers passed the barrier of
+//      step kt - 1), then the loads of slice kt + 2 are issued into the same registers;
+//   2. groups 0..2 of the slice: 16 MFMAs each, the fragments of the next group requested before them;
+//   3. the workgroup barrier sits before the last group, when every LDS read of the step has returned
+//      and the stores of 1. have long completed; right after it the first fragments of slice kt + 1
+//      are requested, so that they arrive under the 16 MFMAs of group 3.
+// No phase of the step is without MFMAs in flight: a wavefront never waits for memory and then for
+// the barrier and then for LDS with the matrix pipe idle.
 template <bool VEC>
 __device__ __forceinline__ void gemm_tile(
     const GemmOperands& g, int tm, int tn, float* lds, WaveAcc& acc
@@ -179,67 +203,93 @@ __device__ __forceinline__ void gemm_tile(
             for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
 
     const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;
-    const int nk_full = VEC ? g.K / GEMM_BK : 0;  // steps that need no guard
+    const int nk_full = VEC ? g.K / GEMM_BK : 0;  // slices that need no guard
+    const int n_full_steps = g.K / GEMM_BK;       // slices whose 32 columns all hold data
 
-    if (nk_full > 0) {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            ra[p] = load_k4<VEC, false>(a_rows[p], 0, g.K);
-            rb[p] = load_k4<VEC, false>(b_rows[p], 0, g.K);
-        }
-    } else {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, ld_k, g.K);
-            rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, ld_k, g.K);
-        }
-    }
-    const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        *reinterpret_cast<floatx4*>(&As[st_off + 32 * p * GEMM_LDS_STRIDE]) = ra[p];
-        *reinterpret_cast<floatx4*>(&Bs[st_off + 32 * p * GEMM_LDS_STRIDE]) = rb[p];
-    }
-    __syncthreads();
-
-    const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
-    const int n_full_steps = g.K / GEMM_BK;  // steps whose 32 columns all hold data
-    for (int kt = 0; kt < n_full_steps; ++kt) {
-        const int cur = kt & 1;
-        const bool more = (kt + 1) < nk;
-        if (more) {
-            const int k0 = (kt + 1) * GEMM_BK;
-            if (kt + 1 < nk_full) {
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
-                    rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
-                }
-            } else {
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
-                    rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
-                }
-            }
-        }
-        mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off,
-                       Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off, acc);
-        if (more) {
-            float* asn = As + (cur ^ 1) * GEMM_TM * GEMM_LDS_STRIDE + st_off;
-            float* bsn = Bs + (cur ^ 1) * GEMM_TN * GEMM_LDS_STRIDE + st_off;
+    auto request = [&](int kt) {  // slice kt -> registers
+        const int k0 = kt * GEMM_BK;
+        if (kt < nk_full) {
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                *reinterpret_cast<floatx4*>(&asn[32 * p * GEMM_LDS_STRIDE]) = ra[p];
-                *reinterpret_cast<floatx4*>(&bsn[32 * p * GEMM_LDS_STRIDE]) = rb[p];
+                ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
+                rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
             }
         }
-        __syncthreads();
-    }
+    };
+    const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
+    auto publish = [&](int buf) {  // registers -> LDS buffer
+        float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + st_off;
+        float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + st_off;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            *reinterpret_cast<floatx4*>(&as[32 * p * GEMM_LDS_STRIDE]) = ra[p];
+            *reinterpret_cast<floatx4*>(&bs[32 * p * GEMM_LDS_STRIDE]) = rb[p];
+        }
+    };
+
+    const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
+    const int a_frag = (wm * 64) * GEMM_LDS_STRIDE + frag_off;
+    const int b_frag = (wn * 64) * GEMM_LDS_STRIDE + frag_off;
+    floatx4 a0, a1, b0, b1;
+    auto fetch = [&](int buf, int kg, floatx4& f0, floatx4& f1, floatx4& g0, floatx4& g1) {
+        const float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + a_frag + kg * 8;
+        const float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + b_frag + kg * 8;
+        f0 = *reinterpret_cast<const floatx4*>(as);
+        f1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
+        g0 = *reinterpret_cast<const floatx4*>(bs);
+        g1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
+    };
+
+    // Prologue: slice 0 in LDS buffer 0, slice 1 (if any) on its way into the registers.
+    request(0);
+    publish(0);
+    if (nk > 1) request(1);
+    __syncthreads();
+    if (n_full_steps > 0) fetch(0, 0, a0, a1, b0, b1);
+
+    // One full step.  HOT: slices kt + 1 and kt + 2 exist and need no guard (no condition in the step).
+    auto step = [&](const int kt, auto hot) {
+        constexpr bool HOT = decltype(hot)::value;
+        const int cur = kt & 1;
+        if (HOT) {
+            publish(cur ^ 1);
+            const int k0 = (kt + 2) * GEMM_BK;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            }
+        } else {
+            if (kt + 1 < nk) publish(cur ^ 1);
+            if (kt + 2 < nk) request(kt + 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        floatx4 na0, na1, nb0, nb1;
+#pragma unroll
+        for (int kg = 0; kg < GEMM_BK / 8 - 1; ++kg) {
+            fetch(cur, kg + 1, na0, na1, nb0, nb1);
+            mfma_group(a0, a1, b0, b1, acc);
+            a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();  // every read of buffer `cur` has returned, slice kt + 1 is complete in the other one
+        if (HOT || kt + 1 < n_full_steps) fetch(cur ^ 1, 0, na0, na1, nb0, nb1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_group(a0, a1, b0, b1, acc);
+        a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+    };
+    int kt = 0;
+    for (; kt + 2 < nk_full; ++kt) step(kt, std::true_type{});
+    for (; kt < n_full_steps; ++kt) step(kt, std::false_type{});
     if (n_full_steps < nk) {
         const int cur = n_full_steps & 1;
-        mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + (wm * 64) * GEMM_LDS_STRIDE + frag_off,
-                       Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + (wn * 64) * GEMM_LDS_STRIDE + frag_off, acc,
+        mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc,
                        (g.K - n_full_steps * GEMM_BK + 7) / 8);
         __syncthreads();
     }

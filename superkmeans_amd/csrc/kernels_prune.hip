@@ -160,24 +160,31 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             } else {
                 xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
             }
-            for (int s0 = 0; s0 < cnt; s0 += 4) {
-                const int s = s0 + grp;
-                const bool in = s < cnt;
-                const int cpos = in ? pos[s] : pos[0];
-                const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
-                float4 cv;
-                if (VEC) {
-                    cv = *reinterpret_cast<const float4*>(cb);
-                } else {
-                    cv = make_float4(cb[0], cb[1], cb[2], cb[3]);
+            // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
+            for (int s0 = 0; s0 < cnt; s0 += 16) {
+                float4 cv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int s = s0 + 4 * u + grp;
+                    const int cpos = s < cnt ? pos[s] : pos[0];
+                    const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                    if (VEC) {
+                        cv[u] = *reinterpret_cast<const float4*>(cb);
+                    } else {
+                        cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
+                    }
                 }
-                float e, part = 0.0f;
-                e = xv.x - cv.x; part += e * e;
-                e = xv.y - cv.y; part += e * e;
-                e = xv.z - cv.z; part += e * e;
-                e = xv.w - cv.w; part += e * e;
-                part = group16_sum(part);
-                if (in && sub == 0) acc[s] += part;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int s = s0 + 4 * u + grp;
+                    float e, part = 0.0f;
+                    e = xv.x - cv[u].x; part += e * e;
+                    e = xv.y - cv[u].y; part += e * e;
+                    e = xv.z - cv[u].z; part += e * e;
+                    e = xv.w - cv[u].w; part += e * e;
+                    part = group16_sum(part);
+                    if (s < cnt && sub == 0) acc[s] += part;
+                }
             }
             dims_seen += SKM_H_DIM_SIZE;
             thr = best * a.ratios[dims_seen];
@@ -393,24 +400,31 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
             } else {
                 xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
             }
-            for (int s0 = 0; s0 < cnt; s0 += 4) {
-                const int s = s0 + grp;
-                const bool in = s < cnt;
-                const int cpos = in ? pos[s] : pos[0];
-                const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
-                float4 cv;
-                if (VEC) {
-                    cv = *reinterpret_cast<const float4*>(cb);
-                } else {
-                    cv = make_float4(cb[0], cb[1], cb[2], cb[3]);
+            // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
+            for (int s0 = 0; s0 < cnt; s0 += 16) {
+                float4 cv[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int s = s0 + 4 * u + grp;
+                    const int cpos = s < cnt ? pos[s] : pos[0];
+                    const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                    if (VEC) {
+                        cv[u] = *reinterpret_cast<const float4*>(cb);
+                    } else {
+                        cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
+                    }
                 }
-                float e, part = 0.0f;
-                e = xv.x - cv.x; part += e * e;
-                e = xv.y - cv.y; part += e * e;
-                e = xv.z - cv.z; part += e * e;
-                e = xv.w - cv.w; part += e * e;
-                part = group16_sum(part);
-                if (in && sub == 0) acc[s] += part;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int s = s0 + 4 * u + grp;
+                    float e, part = 0.0f;
+                    e = xv.x - cv[u].x; part += e * e;
+                    e = xv.y - cv[u].y; part += e * e;
+                    e = xv.z - cv[u].z; part += e * e;
+                    e = xv.w - cv[u].w; part += e * e;
+                    part = group16_sum(part);
+                    if (s < cnt && sub == 0) acc[s] += part;
+                }
             }
             dims_seen += SKM_H_DIM_SIZE;
             thr = best * a.ratios[dims_seen];
