@@ -3,8 +3,10 @@
 // algorithm (batch shapes decide tie-breaking and threshold schedules), not tuning knobs.
 #pragma once
 
+#include <cmath>
 #include <cstddef>
 #include <cstdint>
+#include <random>
 #include <stdexcept>
 #include <string>
 
@@ -34,6 +36,45 @@ static inline constexpr float HIERARCHICAL_PRUNER_INITIAL_THRESHOLD = 1.1f;
 // Kept for source compatibility: host-side loops of this backend are single threaded, the
 // per-point work runs on the device.
 inline uint32_t g_n_threads = 1;
+
+// The value sequence of std::uniform_real_distribution<float>(0, 1)(rng) over a std::mt19937, drawn by the
+// cluster-splitting walk millions of times per call.  With libstdc++ that is one 32-bit draw scaled by 2^-32
+// and kept below 1; the direct form is several times faster than going through generate_canonical.  Whether
+// the two agree is checked once per process on a fixed stream; if they do not (another standard library), every
+// draw goes through the standard distribution, which is what the reference calls.
+class UnitUniformDraws {
+  public:
+    explicit UnitUniformDraws(std::mt19937& rng) : rng_(rng), direct_(DirectFormMatches()) {}
+    float operator()() {
+        if (!direct_) return std::uniform_real_distribution<float>(0, 1)(rng_);
+        const float r = static_cast<float>(rng_()) * 0x1p-32f;
+        return r < 1.0f ? r : std::nextafter(1.0f, 0.0f);
+    }
+
+  private:
+    static bool DirectFormMatches() {
+        static const bool ok = [] {
+            std::mt19937 a(20240229u), b(20240229u);
+            for (int i = 0; i < 1 << 16; ++i) {
+                const float ref = std::uniform_real_distribution<float>(0, 1)(a);
+                float r = static_cast<float>(b()) * 0x1p-32f;
+                if (!(r < 1.0f)) r = std::nextafter(1.0f, 0.0f);
+                if (r != ref) return false;
+            }
+            // the largest draws round up to 2^32 as floats: the clamp must give what the library gives
+            struct Top {
+                using result_type = std::mt19937::result_type;
+                static constexpr result_type min() { return std::mt19937::min(); }
+                static constexpr result_type max() { return std::mt19937::max(); }
+                result_type operator()() { return max(); }
+            } top;
+            return std::uniform_real_distribution<float>(0, 1)(top) == std::nextafter(1.0f, 0.0f);
+        }();
+        return ok;
+    }
+    std::mt19937& rng_;
+    const bool direct_;
+};
 
 enum class DistanceFunction : uint8_t { l2, dp };
 enum class Quantization : uint8_t { f32, u8, f16, bf16 };

@@ -250,17 +250,27 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         auto& sizes = this->cluster_sizes;
         const size_t average_size = n_samples_ / k;
         const size_t threshold_size = static_cast<size_t>(static_cast<float>(average_size) * BALANCING_THRESHOLD);
+        // Acceptance probabilities of the walk, tabulated and refreshed for the two clusters a split changes.
+        const auto accept_probability = [&](const size_t c) -> float {
+            return (sizes[c] - 1.0f) / static_cast<float>(n_samples_ - k);
+        };
+        std::vector<float> prob;
+        UnitUniformDraws draw(rng);
         for (size_t ci = 0; ci < k; ci++) {
             if (sizes[ci] != 0) continue;
+            if (prob.empty()) {
+                prob.resize(k);
+                for (size_t c = 0; c < k; ++c) prob[c] = accept_probability(c);
+            }
             size_t cj;
             for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
-                float p = (sizes[cj] - 1.0f) / static_cast<float>(n_samples_ - k);
-                float r = std::uniform_real_distribution<float>(0, 1)(rng);
-                if (r < p) break;
+                if (draw() < prob[cj]) break;
             }
             edits.push_back({0u, static_cast<uint32_t>(ci), static_cast<uint32_t>(cj), 0.0f});
             sizes[ci] = sizes[cj] / 2;
             sizes[cj] -= sizes[ci];
+            prob[ci] = accept_probability(ci);
+            prob[cj] = accept_probability(cj);
             this->n_split++;
         }
         for (size_t ci = 0; ci < k; ci++) {
@@ -272,8 +282,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
                 if (large_size < average_size) continue;
                 float p = static_cast<float>(large_size - average_size + 1) /
                           static_cast<float>(n_samples_ - average_size * k + k);
-                float r = std::uniform_real_distribution<float>(0, 1)(rng);
-                if (r < p) break;
+                if (draw() < p) break;
             }
             const float wc = std::min(static_cast<float>(csize), CENTER_ADJUSTMENT_WEIGHT);
             edits.push_back({1u, static_cast<uint32_t>(ci), static_cast<uint32_t>(large), wc});

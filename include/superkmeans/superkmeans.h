@@ -486,17 +486,28 @@ class SuperKMeans {
         n_split = 0;
         std::mt19937 rng(config.seed);
         std::vector<RowEdit> edits;
+        // Acceptance probabilities of the walk, tabulated (an empty cluster takes thousands of visits) and
+        // refreshed for the two clusters a split changes; same arithmetic as the reference's expression.
+        const auto accept_probability = [&](const size_t c) -> float {
+            return (cluster_sizes[c] - 1.0) / (float) (n_samples_ - k);
+        };
+        std::vector<float> prob;
+        UnitUniformDraws draw(rng);
         for (size_t ci = 0; ci < k; ci++) {
             if (cluster_sizes[ci] != 0) continue;
+            if (prob.empty()) {
+                prob.resize(k);
+                for (size_t c = 0; c < k; ++c) prob[c] = accept_probability(c);
+            }
             size_t cj;
             for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
-                float p = (cluster_sizes[cj] - 1.0) / (float) (n_samples_ - k);
-                float r = std::uniform_real_distribution<float>(0, 1)(rng);
-                if (r < p) break;
+                if (draw() < prob[cj]) break;
             }
             edits.push_back({0u, static_cast<uint32_t>(ci), static_cast<uint32_t>(cj), 0.0f});
             cluster_sizes[ci] = cluster_sizes[cj] / 2;
             cluster_sizes[cj] -= cluster_sizes[ci];
+            prob[ci] = accept_probability(ci);
+            prob[cj] = accept_probability(cj);
             n_split++;
         }
         ApplyRowEdits(edits);
