@@ -52,6 +52,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Four consecutive floats of a point row (16-byte load when rows are aligned).
+template <bool VEC>
+__device__ __forceinline__ float4 load_x4(const float* p) {
+    if (VEC) return *reinterpret_cast<const float4*>(p);
+    return make_float4(p[0], p[1], p[2], p[3]);
+}
+
 // Keeps the survivors whose accumulated distance is below thr, preserving order. In-place: slot s
 // is rewritten only by elements read from slots >= s, and each step reads before it writes.
 __device__ __forceinline__ int compact_survivors(uint16_t* pos, float* acc, int cnt, float thr, int lane) {
@@ -150,16 +157,14 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
         // ---- horizontal blocks of 64 dimensions, PDX layout (pdxearch.h:149-180) ----
         const float* chunk = a.pdx + (int64_t) base * d;
         int dims_seen = dp;
+        float4 xv_next = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (n_hblocks > 0) xv_next = load_x4<VEC>(xq + V + sub * 4);
         for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
             if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
             const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
-            const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
-            float4 xv;
-            if (VEC) {
-                xv = *reinterpret_cast<const float4*>(xb + sub * 4);
-            } else {
-                xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
-            }
+            // This block's slice of the point was requested one block ago; the next one is requested now.
+            const float4 xv = xv_next;
+            if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
             // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
             for (int s0 = 0; s0 < cnt; s0 += 16) {
                 float4 cv[4];
@@ -334,55 +339,37 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
     float best = a.best0[p];
     uint32_t not_pruned_total = 0;
 
-    // Smallest batch that holds a candidate.
-    uint32_t jb = 0xffffffffu;
-    for (uint32_t s0 = 0; s0 < n_cand; s0 += 64) {
-        const uint32_t s = s0 + lane;
-        if (s < n_cand) {
-            const uint32_t b = list[s].x / SKM_Y_BATCH_SIZE;
-            jb = b < jb ? b : jb;
-        }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const uint32_t o = (uint32_t) __shfl_xor((int) jb, off);
-        jb = o < jb ? o : jb;
-    }
+    // The list is ordered by batch (the producer appends tile after tile and a batch is eight consecutive
+    // tiles), so one forward walk serves every batch: 64 entries are held in registers at a time, `cur` is
+    // the first entry not yet consumed.
+    uint32_t chunk0 = 0, cur = 0;
+    uint2 entry = make_uint2(0xffffffffu, 0u);
+    if (lane < n_cand) entry = list[lane];
 
-    while (jb != 0xffffffffu) {
+    while (cur < n_cand) {
+        const uint32_t jb = (uint32_t) __shfl((int) entry.x, (int) (cur - chunk0)) / SKM_Y_BATCH_SIZE;
         const int base = (int) jb * SKM_Y_BATCH_SIZE;
         const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
         const uint32_t prev_top_1 = best_idx;
         float thr = best * a.ratios[dp];
         int cnt = 0;
-        uint32_t next_jb = 0xffffffffu;
-        for (uint32_t s0 = 0; s0 < n_cand; s0 += 64) {
-            const uint32_t s = s0 + lane;
-            bool keep = false;
-            uint2 e = make_uint2(0u, 0u);
-            if (s < n_cand) {
-                e = list[s];
-                const uint32_t b = e.x / SKM_Y_BATCH_SIZE;
-                if (b == jb) {
-                    keep = __uint_as_float(e.y) < thr;
-                } else if (b > jb && b < next_jb) {
-                    next_jb = b;
-                }
-            }
+        for (;;) {
+            const uint32_t s = chunk0 + lane;
+            const bool mine = s >= cur && s < n_cand && entry.x / SKM_Y_BATCH_SIZE == jb;
+            const bool keep = mine && __uint_as_float(entry.y) < thr;
             const unsigned long long mask = __ballot(keep);
             if (keep) {
                 const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
-                pos[slot] = (uint16_t) (e.x - (uint32_t) base);
-                acc[slot] = __uint_as_float(e.y);
+                pos[slot] = (uint16_t) (entry.x - (uint32_t) base);
+                acc[slot] = __uint_as_float(entry.y);
             }
             cnt += __popcll(mask);
+            cur += (uint32_t) __popcll(__ballot(mine));  // the entries of the batch are consecutive
+            if (cur < chunk0 + 64 || cur >= n_cand) break;  // the batch ended inside this chunk, or the list did
+            chunk0 += 64;
+            entry = make_uint2(0xffffffffu, 0u);
+            if (chunk0 + lane < n_cand) entry = list[chunk0 + lane];
         }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const uint32_t o = (uint32_t) __shfl_xor((int) next_jb, off);
-            next_jb = o < next_jb ? o : next_jb;
-        }
-        jb = next_jb;
         not_pruned_total += (uint32_t) cnt;
         if (acct && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
         if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
@@ -390,16 +377,14 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
 
         const float* chunk = a.pdx + (int64_t) base * d;
         int dims_seen = dp;
+        float4 xv_next = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (n_hblocks > 0) xv_next = load_x4<VEC>(xq + V + sub * 4);
         for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
             if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
             const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
-            const float* xb = xq + V + hb * SKM_H_DIM_SIZE;
-            float4 xv;
-            if (VEC) {
-                xv = *reinterpret_cast<const float4*>(xb + sub * 4);
-            } else {
-                xv = make_float4(xb[sub * 4], xb[sub * 4 + 1], xb[sub * 4 + 2], xb[sub * 4 + 3]);
-            }
+            // This block's slice of the point was requested one block ago; the next one is requested now.
+            const float4 xv = xv_next;
+            if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
             // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
             for (int s0 = 0; s0 < cnt; s0 += 16) {
                 float4 cv[4];
