@@ -16,45 +16,65 @@ constexpr int SORT_THREADS = 256;
 constexpr int SORT_TILE = 4096;  // elements per workgroup and pass
 constexpr int RADIX = 256;
 
-__global__ __launch_bounds__(256) void count_assignments_kernel(
-    const uint32_t* __restrict__ idx, size_t n, uint32_t k, uint32_t* __restrict__ sizes
-) {
-    size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t stride = (size_t) gridDim.x * blockDim.x;
-    for (; i < n; i += stride) {
-        const uint32_t a = idx[i];
-        if (a < k) atomicAdd(&sizes[a], 1u);
-    }
-}
-
-// Exclusive scan of `len` counters by one workgroup (len is k + 1 or 256 * n_tiles: small).
+// Exclusive scan of `len` counters by one workgroup (len is 256 * n_tiles: a few hundred KB at most).
+// Each of the 16 wavefronts owns a contiguous segment: it adds the segment up with coalesced loads, the 16
+// totals are exchanged through LDS (the only barrier), then the wavefront scans its segment 64 counters at a
+// time with shuffles, carrying the running total in a register.
 __global__ __launch_bounds__(1024) void exclusive_scan_kernel(
     const uint32_t* __restrict__ in, uint32_t* __restrict__ out, size_t len
 ) {
     __shared__ uint32_t s_wave[16];
-    __shared__ uint32_t s_carry;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) s_carry = 0;
+    const size_t seg = ((len + 15) / 16 + 63) / 64 * 64;
+    const size_t begin = (size_t) wave * seg < len ? (size_t) wave * seg : len;
+    const size_t end = begin + seg < len ? begin + seg : len;
+    uint32_t total = 0;
+#pragma unroll 8
+    for (size_t i = begin + lane; i < end; i += 64) total += in[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    if (lane == 0) s_wave[wave] = total;
     __syncthreads();
-    for (size_t base = 0; base < len; base += 1024) {
-        const size_t i = base + tid;
-        const uint32_t v = (i < len) ? in[i] : 0u;
+    uint32_t carry = 0;
+    for (int w = 0; w < wave; ++w) carry += s_wave[w];
+#pragma unroll 4
+    for (size_t base = begin; base < end; base += 64) {
+        const size_t i = base + lane;
+        const uint32_t v = i < end ? in[i] : 0u;
         uint32_t incl = v;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const uint32_t t = __shfl_up(incl, off);
             if (lane >= off) incl += t;
         }
-        if (lane == 63) s_wave[wave] = incl;
-        __syncthreads();
-        uint32_t wave_off = 0;
-        for (int w = 0; w < wave; ++w) wave_off += s_wave[w];
-        const uint32_t carry = s_carry;
-        if (i < len) out[i] = carry + wave_off + incl - v;
-        __syncthreads();
-        if (tid == 1023) s_carry = carry + wave_off + incl;
-        __syncthreads();
+        if (i < end) out[i] = carry + incl - v;
+        carry += __shfl(incl, 63);
     }
+}
+
+// Segment boundaries of the sorted assignment keys: offsets[c] = first position whose key is >= c
+// (offsets[k] = number of keys below k), written by the thread that sees the key change.
+__global__ __launch_bounds__(256) void segment_bounds_kernel(
+    const uint32_t* __restrict__ sorted_keys, size_t n, uint32_t k, uint32_t* __restrict__ offsets
+) {
+    const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i > n) return;
+    // Position n closes the last segment: it behaves like a key equal to k.
+    uint32_t key = i < n ? sorted_keys[i] : k;
+    key = key < k ? key : k;
+    uint32_t first = 0;
+    if (i > 0) {
+        const uint32_t prev = sorted_keys[i - 1];
+        first = (prev < k ? prev : k) + 1;
+    }
+    for (uint32_t c = first; c <= key; ++c) offsets[c] = (uint32_t) i;
+}
+
+__global__ __launch_bounds__(256) void sizes_from_offsets_kernel(
+    const uint32_t* __restrict__ offsets, uint32_t k, uint32_t* __restrict__ sizes
+) {
+    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < k) sizes[c] = offsets[c + 1] - offsets[c];
 }
 
 // Pass 1 of a radix step: digit histogram of one tile, stored digit-major so that one exclusive
@@ -323,22 +343,6 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     uint32_t* hist = offsets + (k + 1);
     uint32_t* bases = hist + hist_len;
 
-    SKM_TRY(skm_fill_u32(ctx, d_out_sizes, 0u, k));
-    if (n > 0) {
-        const unsigned blocks = (unsigned) std::min<size_t>((n + 255) / 256, 4096);
-        hipLaunchKernelGGL(count_assignments_kernel, dim3(blocks), dim3(256), 0, ctx->stream, d_idx, n, (uint32_t) k, d_out_sizes);
-        SKM_HIP_TRY(hipGetLastError());
-    }
-    // offsets[c] = number of points assigned to centroids < c and offsets[k] = n: exclusive scan of
-    // the sizes followed by one zero.
-    void* ws2 = nullptr;
-    SKM_TRY(workspace(ctx, 2, (k + 1) * sizeof(uint32_t), &ws2));
-    uint32_t* sizes_z = (uint32_t*) ws2;
-    SKM_HIP_TRY(hipMemcpyAsync(sizes_z, d_out_sizes, k * sizeof(uint32_t), hipMemcpyDeviceToDevice, ctx->stream));
-    SKM_TRY(skm_fill_u32(ctx, sizes_z + k, 0u, 1));
-    hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, sizes_z, offsets, k + 1);
-    SKM_HIP_TRY(hipGetLastError());
-
     const uint32_t* sorted_ids = nullptr;
     if (n > 0) {
         int bits = 0;
@@ -363,9 +367,17 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
             vout = (vout == vals_a) ? vals_b : vals_a;
         }
         sorted_ids = vin;
+        // Sizes and segment offsets come from the sorted keys: no counting pass over the assignments.
+        hipLaunchKernelGGL(segment_bounds_kernel, dim3((unsigned) ((n + 1 + 255) / 256)), dim3(256), 0, ctx->stream, kin, n,
+                           (uint32_t) k, offsets);
+        SKM_HIP_TRY(hipGetLastError());
     } else {
         sorted_ids = vals_a;
+        SKM_TRY(skm_fill_u32(ctx, offsets, 0u, k + 1));
     }
+    hipLaunchKernelGGL(sizes_from_offsets_kernel, dim3((unsigned) ((k + 255) / 256)), dim3(256), 0, ctx->stream, offsets,
+                       (uint32_t) k, d_out_sizes);
+    SKM_HIP_TRY(hipGetLastError());
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
     const size_t lanes = vec ? d / 4 : d;
