@@ -162,13 +162,26 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(
         for (size_t t = threadIdx.x; t < d4; t += blockDim.x) {
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
             uint32_t j = j0;
-            for (; j + 8 <= j1; j += 8) {
-                float4 v[8];
+            for (; j + 16 <= j1; j += 16) {
+                float4 v[16];
 #pragma unroll
-                for (int u = 0; u < 8; ++u)
+                for (int u = 0; u < 16; ++u)
                     v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) {
+                for (int u = 0; u < 16; ++u) {
+                    acc.x += v[u].x;
+                    acc.y += v[u].y;
+                    acc.z += v[u].z;
+                    acc.w += v[u].w;
+                }
+            }
+            for (; j + 4 <= j1; j += 4) {
+                float4 v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
                     acc.x += v[u].x;
                     acc.y += v[u].y;
                     acc.z += v[u].z;
