@@ -10,6 +10,10 @@
 //   3. refinement: optional pruned iterations over all k clusters.
 #pragma once
 
+#include <atomic>
+#include <exception>
+#include <thread>
+
 #include "superkmeans/superkmeans.h"
 
 namespace skmeans {
@@ -41,9 +45,9 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
   public:
     HierarchicalSuperKMeans(size_t n_clusters, size_t dimensionality, const HierarchicalSuperKMeansConfig& config)
         : base(n_clusters, dimensionality, config), hierarchical_config(config) {
-        // Looser ADSampling epsilon for the hierarchical driver (common.h of the reference, :115).
-        this->pruner = std::make_unique<pruner_t>(this->ctx, dimensionality, HIERARCHICAL_PRUNER_INITIAL_THRESHOLD,
-                                                  this->config.seed);
+        // Looser ADSampling epsilon for the hierarchical driver (common.h of the reference, :115): same
+        // rotation matrix (same seed), other threshold ratios.
+        this->pruner->SetEpsilon0(HIERARCHICAL_PRUNER_INITIAL_THRESHOLD);
         SKMEANS_ENSURE_POSITIVE(config.iters_mesoclustering);
         SKMEANS_ENSURE_POSITIVE(config.iters_fineclustering);
         static_cast<SuperKMeansConfig&>(hierarchical_config) = this->config;
@@ -57,6 +61,14 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
 
     HierarchicalSuperKMeans(size_t n_clusters, size_t dimensionality)
         : HierarchicalSuperKMeans(n_clusters, dimensionality, HierarchicalSuperKMeansConfig{}) {}
+
+  protected:
+    // Fine-phase helper of `owner`: own device context, the owner's pruner tables and configuration.
+    struct FineHelperTag {};
+    HierarchicalSuperKMeans(const HierarchicalSuperKMeans& owner, FineHelperTag)
+        : base(owner.n_clusters, owner.d, owner.config, owner.pruner), hierarchical_config(owner.hierarchical_config) {}
+
+  public:
 
     /** Hierarchical training on host-resident data; queries are ignored (as in the reference). */
     std::vector<centroid_value_t> Train(const vector_value_t* data, const size_t n,
@@ -153,31 +165,63 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
                       << k << " clusters) ===" << std::endl;
         const auto fine_clusters_nums = ArrangeFineClusters(k, n_mesoclusters, total_samples, mesoclusters_sizes);
         const size_t max_mesocluster_size = *std::max_element(mesoclusters_sizes.begin(), mesoclusters_sizes.end());
-        dbuf<float> mesocluster_buffer(ctx, std::max<size_t>(1, max_mesocluster_size) * d);
-        size_t fineclusters_offset = 0;
+        const size_t max_fineclusters = *std::max_element(fine_clusters_nums.begin(), fine_clusters_nums.end());
+        std::vector<size_t> fine_offsets(n_mesoclusters + 1, 0);
+        for (size_t m = 0; m < n_mesoclusters; ++m) fine_offsets[m + 1] = fine_offsets[m] + fine_clusters_nums[m];
+        FineInputs in;
+        in.data_to_cluster = data_to_cluster;
+        in.full_norms = immutable_data_norms.get();
+        in.member_ids = d_indices.get();
+        in.member_offsets = offsets.data();
+        in.sizes = mesoclusters_sizes.data();
+        in.fine_counts = fine_clusters_nums.data();
+        in.fine_offsets = fine_offsets.data();
+        in.initial_partial_d = initial_partial_d;
+        in.out_assignments = final_assignments.get();
+        in.out_centroids = final_centroids.get();
+        // The mesoclusters are independent problems of a few thousand points each, far too small to fill the
+        // device one at a time: several helpers, each with its own stream and scratch, take them from a common
+        // counter.  Every problem is computed exactly as it would be alone; the statistics are put back in
+        // mesocluster order afterwards.
+        std::vector<std::vector<SuperKMeansIterationStats>> fine_stats(n_mesoclusters);
+        const size_t wanted = this->config.n_threads == 0 ? FINE_HELPERS_DEFAULT : this->config.n_threads;
+        const size_t n_helpers = std::max<size_t>(1, std::min<size_t>({wanted, FINE_HELPERS_MAX, n_mesoclusters}));
+        hip::Check(skm_sync(ctx));  // everything the helpers read is complete
+        if (n_helpers == 1) {
+            dbuf<float> mesocluster_buffer(ctx, std::max<size_t>(1, max_mesocluster_size) * d);
+            for (size_t m = 0; m < n_mesoclusters; ++m) FineClusterOne(in, m, mesocluster_buffer.get(), fine_stats[m]);
+        } else {
+            std::vector<std::unique_ptr<HierarchicalSuperKMeans>> helpers;
+            for (size_t h = 0; h < n_helpers; ++h) {
+                helpers.emplace_back(new HierarchicalSuperKMeans(*this, FineHelperTag{}));
+                helpers.back()->n_samples = std::max<size_t>(1, max_mesocluster_size);  // sizes the per-point buffers
+                helpers.back()->AllocateState(std::max<size_t>(1, max_mesocluster_size), std::max<size_t>(1, max_fineclusters));
+            }
+            std::atomic<size_t> next{0};
+            std::vector<std::exception_ptr> failures(n_helpers);
+            std::vector<std::thread> threads;
+            for (size_t h = 0; h < n_helpers; ++h) {
+                threads.emplace_back([&, h] {
+                    try {
+                        HierarchicalSuperKMeans& helper = *helpers[h];
+                        dbuf<float> buffer(helper.ctx, std::max<size_t>(1, max_mesocluster_size) * d);
+                        for (size_t m = next.fetch_add(1); m < n_mesoclusters; m = next.fetch_add(1)) {
+                            helper.FineClusterOne(in, m, buffer.get(), fine_stats[m]);
+                        }
+                        hip::Check(skm_sync(helper.ctx));
+                    } catch (...) {
+                        failures[h] = std::current_exception();
+                        next.store(n_mesoclusters);  // the others stop taking work
+                    }
+                });
+            }
+            for (auto& t : threads) t.join();
+            for (auto& f : failures)
+                if (f) std::rethrow_exception(f);
+        }
         for (size_t m = 0; m < n_mesoclusters; ++m) {
-            const size_t n_fineclusters = fine_clusters_nums[m];
-            if (n_fineclusters == 0) continue;
-            this->partial_d = initial_partial_d;
-            const size_t mesocluster_size = mesoclusters_sizes[m];
-            this->n_samples = mesocluster_size;
-            const uint64_t* d_member_ids = d_indices.get() + offsets[m];
-            // Rows and full norms of the members, contiguous (CompactMesoclusterToBuffer).
-            hip::Check(skm_gather_rows(ctx, data_to_cluster, d, d_member_ids, mesocluster_size, mesocluster_buffer.get(),
-                                       immutable_data_norms.get(), this->data_norms.get()));
-            this->GenerateCentroids(mesocluster_buffer.get(), mesocluster_size, n_fineclusters, /*rotate=*/false,
-                                    /*on_device=*/true);
-            hip::Check(skm_copy(ctx, this->prev_centroids.get(), this->horizontal_centroids.get(),
-                                sizeof(float) * n_fineclusters * d));
-            RunPhase(hierarchical_config.iters_fineclustering, mesocluster_buffer.get(), mesocluster_size, n_fineclusters,
-                     hierarchical_config.use_blas_only, /*first_iteration_exact=*/true,
-                     hierarchical_iteration_stats.fineclustering_iteration_stats,
-                     hierarchical_config.early_termination);
-            hip::Check(skm_scatter_assignments(ctx, d_member_ids, this->d_assignments.get(), mesocluster_size,
-                                               static_cast<uint32_t>(fineclusters_offset), final_assignments.get()));
-            hip::Check(skm_copy(ctx, final_centroids.get() + fineclusters_offset * d, this->horizontal_centroids.get(),
-                                sizeof(float) * n_fineclusters * d));
-            fineclusters_offset += n_fineclusters;
+            auto& all = hierarchical_iteration_stats.fineclustering_iteration_stats;
+            all.insert(all.end(), fine_stats[m].begin(), fine_stats[m].end());
         }
 
         // ---- phase 3: refinement over all k clusters ----
@@ -207,6 +251,50 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         this->trained = true;
         this->PublishAssignments(total_samples);
         return this->GetOutputCentroids(hierarchical_config.unrotate_centroids);
+    }
+
+    static constexpr size_t FINE_HELPERS_DEFAULT = 4;  // concurrent fine-phase problems when n_threads is 0
+    static constexpr size_t FINE_HELPERS_MAX = 16;
+
+    // What every fine-phase problem reads (device pointers of the owner, host tables) and where it writes.
+    struct FineInputs {
+        const float* data_to_cluster = nullptr;   // rotated samples
+        const float* full_norms = nullptr;         // their norms over all d
+        const uint64_t* member_ids = nullptr;      // sample ids grouped by mesocluster
+        const size_t* member_offsets = nullptr;    // start of every group in member_ids
+        const uint32_t* sizes = nullptr;           // points per mesocluster
+        const size_t* fine_counts = nullptr;       // fine clusters per mesocluster
+        const size_t* fine_offsets = nullptr;      // first global cluster id of every mesocluster
+        uint32_t initial_partial_d = 0;
+        uint32_t* out_assignments = nullptr;       // global cluster id of every sample
+        float* out_centroids = nullptr;            // k x d
+    };
+
+    // Fine clustering of mesocluster m on this object's context (reference hierarchical_superkmeans.h:300-440):
+    // members gathered into `buffer`, Forgy seeding inside the mesocluster, iters_fineclustering iterations,
+    // local ids scattered back with the mesocluster's cluster offset.
+    void FineClusterOne(const FineInputs& in, const size_t m, float* buffer,
+                        std::vector<SuperKMeansIterationStats>& stats) {
+        const size_t n_fineclusters = in.fine_counts[m];
+        if (n_fineclusters == 0) return;
+        const size_t dd = this->d;
+        this->partial_d = in.initial_partial_d;
+        const size_t mesocluster_size = in.sizes[m];
+        this->n_samples = mesocluster_size;
+        const uint64_t* d_member_ids = in.member_ids + in.member_offsets[m];
+        // Rows and full norms of the members, contiguous (CompactMesoclusterToBuffer).
+        hip::Check(skm_gather_rows(this->ctx, in.data_to_cluster, dd, d_member_ids, mesocluster_size, buffer,
+                                   in.full_norms, this->data_norms.get()));
+        this->GenerateCentroids(buffer, mesocluster_size, n_fineclusters, /*rotate=*/false, /*on_device=*/true);
+        hip::Check(skm_copy(this->ctx, this->prev_centroids.get(), this->horizontal_centroids.get(),
+                            sizeof(float) * n_fineclusters * dd));
+        RunPhase(hierarchical_config.iters_fineclustering, buffer, mesocluster_size, n_fineclusters,
+                 hierarchical_config.use_blas_only, /*first_iteration_exact=*/true, stats,
+                 hierarchical_config.early_termination);
+        hip::Check(skm_scatter_assignments(this->ctx, d_member_ids, this->d_assignments.get(), mesocluster_size,
+                                           static_cast<uint32_t>(in.fine_offsets[m]), in.out_assignments));
+        hip::Check(skm_copy(this->ctx, in.out_centroids + in.fine_offsets[m] * dd, this->horizontal_centroids.get(),
+                            sizeof(float) * n_fineclusters * dd));
     }
 
     // Iterations of one phase: the first is always exact (GEMM only); the others are pruned unless the

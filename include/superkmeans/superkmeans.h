@@ -128,12 +128,26 @@ class SuperKMeans {
         g_n_threads = n_threads;
         context = std::make_shared<hip::Context>(0);
         ctx = context->get();
-        pruner = std::make_unique<pruner_t>(ctx, dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed,
+        pruner = std::make_shared<pruner_t>(ctx, dimensionality, PRUNER_INITIAL_THRESHOLD, config.seed,
                                             config.dct_rotation);
         if (this->config.data_already_rotated) {
             this->config.unrotate_centroids = false;
         }
     }
+
+  protected:
+    // A helper object for concurrent sub-problems of another object: its own device context (stream,
+    // scratch), the owner's pruner tables (building the rotation matrix again would cost O(d^3) on the host).
+    SuperKMeans(size_t n_clusters, size_t dimensionality, const SuperKMeansConfig& config,
+                std::shared_ptr<pruner_t> shared_pruner)
+        : d(dimensionality), n_clusters(n_clusters), config(config) {
+        n_threads = 1;
+        context = std::make_shared<hip::Context>(0);
+        ctx = context->get();
+        pruner = std::move(shared_pruner);
+    }
+
+  public:
 
     SuperKMeans(size_t n_clusters, size_t dimensionality)
         : SuperKMeans(n_clusters, dimensionality, SuperKMeansConfig{}) {}
@@ -809,7 +823,7 @@ class SuperKMeans {
 
     std::shared_ptr<hip::Context> context;
     skm_ctx* ctx = nullptr;
-    std::unique_ptr<pruner_t> pruner;
+    std::shared_ptr<pruner_t> pruner;
 
     // Device state (names follow the reference's members, superkmeans.h:1470-1480)
     dbuf<float> centroids;                     // PDX layout

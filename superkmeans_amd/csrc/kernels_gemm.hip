@@ -18,11 +18,9 @@ static int allow_large_lds(Kernel kernel, size_t bytes) {
 
 #define SKM_LAUNCH_GEMM(kernel, grid, block, lds_bytes, stream, ...)                               \
     do {                                                                                           \
-        static bool configured = false;                                                            \
-        if (!configured) {                                                                         \
-            SKM_TRY(allow_large_lds(kernel, lds_bytes));                                           \
-            configured = true;                                                                     \
-        }                                                                                          \
+        /* once per kernel and process; the initialisation of a local static is thread safe */    \
+        static const int lds_rc = allow_large_lds(kernel, lds_bytes);                              \
+        SKM_TRY(lds_rc);                                                                           \
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, __VA_ARGS__);                   \
     } while (0)
 

@@ -29,7 +29,6 @@ __global__ __launch_bounds__(1024) void exclusive_scan_kernel(
     const size_t begin = (size_t) wave * seg < len ? (size_t) wave * seg : len;
     const size_t end = begin + seg < len ? begin + seg : len;
     uint32_t total = 0;
-#pragma unroll 8
     for (size_t i = begin + lane; i < end; i += 64) total += in[i];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off);
