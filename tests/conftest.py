@@ -55,3 +55,21 @@ def make_blobs(n, d, k, std=0.3, seed=0, normalize=True, center_scale=1.0):
 @pytest.fixture(scope="session")
 def blobs():
     return make_blobs
+
+
+GOLDEN_WCSS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "wcss_ground_truth.json")
+
+
+@pytest.fixture(scope="session")
+def golden():
+    """WCSS tables held by the reference's tests (tests/test_wcss.cpp:25-59, test_hierarchical_superkmeans.cpp:636-670)."""
+    import json
+
+    with open(GOLDEN_WCSS) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="session")
+def golden_data(oracle):
+    """The data the tables were made on, regenerated (tests/generate_wcss_ground_truth.cpp:15-31)."""
+    return oracle.make_blobs(10000, 768, 500, False, 0.25, 5.0, 42)

@@ -4,13 +4,8 @@ The oracle restates the reference's algorithm; nothing here retypes the oracle's
 check is either a golden table / property the reference's own tests hold, a closed form or hand-derived
 value, an independent fp64 numpy computation, or an invariant the mathematics fixes.
 """
-import json
-import os
-
 import numpy as np
 import pytest
-
-GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "wcss_ground_truth.json")
 
 
 # ---- PDXLayout::GetDimensionSplit (pdx/layout.h:115-140) ----
@@ -277,16 +272,6 @@ def test_arrange_fine_clusters_and_mesoclusters(oracle):
 
 
 # ---- whole Train(): reference golden WCSS tables and behavioural contract ----
-@pytest.fixture(scope="module")
-def golden():
-    return json.load(open(GOLDEN))
-
-
-@pytest.fixture(scope="module")
-def golden_data(oracle):
-    return oracle.make_blobs(10000, 768, 500, False, 0.25, 5.0, 42)
-
-
 def test_make_blobs_shape_statistics(golden_data):
     X = golden_data
     assert X.shape == (10000, 768) and np.isfinite(X).all()
