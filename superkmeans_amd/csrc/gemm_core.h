@@ -4,16 +4,19 @@
 // exactly the shape of every dense product on the Super K-Means hot path:
 //   * distances  x . c     (reference: batch_computers.h:47-83, sgemm_('T','N'))
 //   * rotation   X . Q^T   (reference: pdx/adsampling.h:191-215)
-// One workgroup (256 threads = 4 wavefronts of 64) owns a 128 x 128 tile of D,
-// each wavefront a 64 x 64 quadrant held as 2 x 2 accumulators of the
-// v_mfma_f32_32x32x2_f32 instruction.  Operand slices of BK = 32 columns are
-// staged through LDS (double buffered, row stride 36 floats so that both the
-// 16-byte stores and the 16-byte fragment reads are bank-conflict free).
+// A workgroup owns one tile of D and each of its wavefronts a block of FM x FN accumulators of the
+// v_mfma_f32_32x32x2_f32 instruction.  Two shapes are built:
+//   * 128 x 128, 4 wavefronts of 64 x 64, two workgroups per CU   (small problems, fused candidate kernel)
+//   * 256 x 256, 8 wavefronts of 128 x 64, one workgroup per CU   (large problems: per MFMA half the global
+//     loads, LDS stores and barriers and three quarters of the fragment reads of the small shape)
+// Operand slices of BK = 32 columns are staged through LDS (double buffered, row stride 36 floats so
+// that both the 16-byte stores and the 16-byte fragment reads are bank-conflict free).
 //
 // The k index inside a group of 8 columns is permuted so that one ds_read_b128
 // per operand fragment feeds four consecutive MFMAs: lane l supplies columns
 // (l / 32) * 4 + i to the i-th MFMA for both A and B, which is a valid GEMM
-// because A and B use the same permutation.
+// because A and B use the same permutation.  The order in which the products of one output element are
+// accumulated does not depend on the tile shape, so both shapes give bit-identical results.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -26,12 +29,31 @@ namespace skm {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int GEMM_TM = 128;
-constexpr int GEMM_TN = 128;
 constexpr int GEMM_BK = 32;
 constexpr int GEMM_LDS_STRIDE = GEMM_BK + 4;
-constexpr int GEMM_THREADS = 256;
 constexpr int GEMM_XCDS = 8;
+
+// WM x WN wavefronts, each FM x FN accumulator blocks of 32 x 32.
+template <int WM_, int WN_, int FM_, int FN_, int WG_PER_CU_>
+struct GemmShape {
+    static constexpr int WM = WM_, WN = WN_, FM = FM_, FN = FN_, WG_PER_CU = WG_PER_CU_;
+    static constexpr int THREADS = WM * WN * 64;
+    static constexpr int TM = WM * FM * 32;
+    static constexpr int TN = WN * FN * 32;
+    static constexpr int WAVE_M = FM * 32;            // rows of D per wavefront
+    static constexpr int WAVE_N = FN * 32;
+    static constexpr int ROWS_PER_LOAD = THREADS / 8;  // operand rows covered by one 16-byte load per thread
+    static constexpr int NLA = TM / ROWS_PER_LOAD;     // loads per thread and slice, A operand
+    static constexpr int NLB = TN / ROWS_PER_LOAD;
+    static constexpr int LDS_FLOATS = 2 * (TM + TN) * GEMM_LDS_STRIDE;
+    static_assert(TM % ROWS_PER_LOAD == 0 && TN % ROWS_PER_LOAD == 0, "tile rows must split evenly over the loads");
+};
+using GemmSmall = GemmShape<2, 2, 2, 2, 2>;
+using GemmBig = GemmShape<2, 4, 4, 2, 1>;
+
+constexpr int GEMM_TM = GemmSmall::TM;
+constexpr int GEMM_TN = GemmSmall::TN;
+constexpr int GEMM_THREADS = GemmSmall::THREADS;
 
 struct GemmOperands {
     const float* A;  // M x K, row stride lda
@@ -41,13 +63,15 @@ struct GemmOperands {
     int tiles_m, tiles_n;
 };
 
-// Accumulators of one wavefront: acc[mb][nb] is a 32 x 32 block.  Element r of
+// Accumulators of one wavefront: acc.v[mb][nb] is a 32 x 32 block.  Element r of
 // acc[mb][nb] held by lane l is D[m][n] with
 //   m = wave_m0 + mb * 32 + 8 * (r / 4) + 4 * (l / 32) + (r % 4)
 //   n = wave_n0 + nb * 32 + (l % 32)
-struct WaveAcc {
-    floatx16 v[2][2];
+template <int FM, int FN>
+struct WaveAccT {
+    floatx16 v[FM][FN];
 };
+using WaveAcc = WaveAccT<2, 2>;
 
 __device__ __forceinline__ int acc_row(int mb, int r, int lane) {
     return mb * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
@@ -155,50 +179,55 @@ __device__ __forceinline__ void mfma_group(const floatx4& a0, const floatx4& a1,
     }
 }
 
-// Computes the 128 x 128 tile (tm, tn).  VEC: row starts and strides are 16-byte aligned so operand
+// Computes the tile (tm, tn) of shape S.  VEC: row starts and strides are 16-byte aligned so operand
 // slices can be fetched with dwordx4 loads; then every full BK step is fetched without any guard (the
-// eight loads of a thread are issued back to back) and only a trailing partial step is guarded.
+// loads of a thread are issued back to back) and only a trailing partial step is guarded.
 //
 // Schedule of one full step kt (LDS buffer kt & 1 holds slice kt, registers hold slice kt + 1):
 //   1. slice kt + 1 goes from registers to the other LDS buffer (its last readers passed the barrier of
 //      step kt - 1), then the loads of slice kt + 2 are issued into the same registers;
-//   2. groups 0..2 of the slice: 16 MFMAs each, the fragments of the next group requested before them;
+//   2. groups 0..2 of the slice: FM * FN * 4 MFMAs each, the fragments of the next group requested before them;
 //   3. the workgroup barrier sits before the last group, when every LDS read of the step has returned
 //      and the stores of 1. have long completed; right after it the first fragments of slice kt + 1
-//      are requested, so that they arrive under the 16 MFMAs of group 3.
+//      are requested, so that they arrive under the MFMAs of group 3.
 // No phase of the step is without MFMAs in flight: a wavefront never waits for memory and then for
 // the barrier and then for LDS with the matrix pipe idle.
-template <bool VEC>
+template <bool VEC, class S>
 __device__ __forceinline__ void gemm_tile(
-    const GemmOperands& g, int tm, int tn, float* lds, WaveAcc& acc
+    const GemmOperands& g, int tm, int tn, float* lds, WaveAccT<S::FM, S::FN>& acc
 ) {
-    float* As = lds;                                    // [2][TM * STRIDE]
-    float* Bs = lds + 2 * GEMM_TM * GEMM_LDS_STRIDE;    // [2][TN * STRIDE]
+    constexpr int FM = S::FM, FN = S::FN;
+    float* As = lds;                                  // [2][TM * STRIDE]
+    float* Bs = lds + 2 * S::TM * GEMM_LDS_STRIDE;    // [2][TN * STRIDE]
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / S::WN, wn = wave % S::WN;
 
-    // Global -> register staging: thread covers rows (tid / 8) + 32 * p, 4 floats at column 4 * (tid % 8).
+    // Global -> register staging: thread covers rows (tid / 8) + ROWS_PER_LOAD * p, 4 floats at column 4 * (tid % 8).
+    // Rows past the end are clamped to the last row: duplicates are masked by the epilogue.
     const int ld_row = tid >> 3;
     const int ld_k = (tid & 7) * 4;
-    const float* a_rows[4];
-    const float* b_rows[4];
+    const float* a_rows[S::NLA];
+    const float* b_rows[S::NLB];
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        int ra = tm * GEMM_TM + ld_row + 32 * p;
-        int rb = tn * GEMM_TN + ld_row + 32 * p;
-        ra = ra < g.M ? ra : g.M - 1;  // clamp: duplicates are masked by the epilogue
-        rb = rb < g.N ? rb : g.N - 1;
-        a_rows[p] = g.A + (int64_t) ra * g.lda + ld_k;
-        b_rows[p] = g.B + (int64_t) rb * g.ldb + ld_k;
+    for (int p = 0; p < S::NLA; ++p) {
+        int r = tm * S::TM + ld_row + S::ROWS_PER_LOAD * p;
+        r = r < g.M ? r : g.M - 1;
+        a_rows[p] = g.A + (int64_t) r * g.lda + ld_k;
     }
-    floatx4 ra[4], rb[4];
+#pragma unroll
+    for (int p = 0; p < S::NLB; ++p) {
+        int r = tn * S::TN + ld_row + S::ROWS_PER_LOAD * p;
+        r = r < g.N ? r : g.N - 1;
+        b_rows[p] = g.B + (int64_t) r * g.ldb + ld_k;
+    }
+    floatx4 ra[S::NLA], rb[S::NLB];
 
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < FM; ++mb)
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
+        for (int nb = 0; nb < FN; ++nb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
 
@@ -210,40 +239,53 @@ __device__ __forceinline__ void gemm_tile(
         const int k0 = kt * GEMM_BK;
         if (kt < nk_full) {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
-                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
-            }
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+#pragma unroll
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
         } else {
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
-                rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
-            }
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
+#pragma unroll
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
         }
     };
     const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
     auto publish = [&](int buf) {  // registers -> LDS buffer
-        float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + st_off;
-        float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + st_off;
+        float* as = As + buf * S::TM * GEMM_LDS_STRIDE + st_off;
+        float* bs = Bs + buf * S::TN * GEMM_LDS_STRIDE + st_off;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            *reinterpret_cast<floatx4*>(&as[32 * p * GEMM_LDS_STRIDE]) = ra[p];
-            *reinterpret_cast<floatx4*>(&bs[32 * p * GEMM_LDS_STRIDE]) = rb[p];
-        }
+        for (int p = 0; p < S::NLA; ++p) *reinterpret_cast<floatx4*>(&as[S::ROWS_PER_LOAD * p * GEMM_LDS_STRIDE]) = ra[p];
+#pragma unroll
+        for (int p = 0; p < S::NLB; ++p) *reinterpret_cast<floatx4*>(&bs[S::ROWS_PER_LOAD * p * GEMM_LDS_STRIDE]) = rb[p];
     };
 
     const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
-    const int a_frag = (wm * 64) * GEMM_LDS_STRIDE + frag_off;
-    const int b_frag = (wn * 64) * GEMM_LDS_STRIDE + frag_off;
-    floatx4 a0, a1, b0, b1;
-    auto fetch = [&](int buf, int kg, floatx4& f0, floatx4& f1, floatx4& g0, floatx4& g1) {
-        const float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + a_frag + kg * 8;
-        const float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + b_frag + kg * 8;
-        f0 = *reinterpret_cast<const floatx4*>(as);
-        f1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
-        g0 = *reinterpret_cast<const floatx4*>(bs);
-        g1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
+    const int a_frag = (wm * S::WAVE_M) * GEMM_LDS_STRIDE + frag_off;
+    const int b_frag = (wn * S::WAVE_N) * GEMM_LDS_STRIDE + frag_off;
+    floatx4 fa[FM], fb[FN];
+    auto fetch = [&](int buf, int kg, floatx4* xa, floatx4* xb) {
+        const float* as = As + buf * S::TM * GEMM_LDS_STRIDE + a_frag + kg * 8;
+        const float* bs = Bs + buf * S::TN * GEMM_LDS_STRIDE + b_frag + kg * 8;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) xa[i] = *reinterpret_cast<const floatx4*>(as + i * 32 * GEMM_LDS_STRIDE);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) xb[j] = *reinterpret_cast<const floatx4*>(bs + j * 32 * GEMM_LDS_STRIDE);
+    };
+    // The FM * FN * 4 MFMAs of one group of 8 columns; consecutive MFMAs never share an accumulator.
+    auto group = [&]() {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc.v[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][q], fb[j][q], acc.v[i][j], 0, 0, 0);
+    };
+    auto advance = [&](const floatx4* na, const floatx4* nb) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) fa[i] = na[i];
+#pragma unroll
+        for (int j = 0; j < FN; ++j) fb[j] = nb[j];
     };
 
     // Prologue: slice 0 in LDS buffer 0, slice 1 (if any) on its way into the registers.
@@ -251,7 +293,7 @@ __device__ __forceinline__ void gemm_tile(
     publish(0);
     if (nk > 1) request(1);
     __syncthreads();
-    if (n_full_steps > 0) fetch(0, 0, a0, a1, b0, b1);
+    if (n_full_steps > 0) fetch(0, 0, fa, fb);
 
     // One full step.  HOT: slices kt + 1 and kt + 2 exist and need no guard (no condition in the step).
     auto step = [&](const int kt, auto hot) {
@@ -261,41 +303,47 @@ __device__ __forceinline__ void gemm_tile(
             publish(cur ^ 1);
             const int k0 = (kt + 2) * GEMM_BK;
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
-                rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
-            }
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+#pragma unroll
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
         } else {
             if (kt + 1 < nk) publish(cur ^ 1);
             if (kt + 2 < nk) request(kt + 2);
         }
         __builtin_amdgcn_sched_barrier(0);
-        floatx4 na0, na1, nb0, nb1;
+        floatx4 na[FM], nb[FN];
 #pragma unroll
         for (int kg = 0; kg < GEMM_BK / 8 - 1; ++kg) {
-            fetch(cur, kg + 1, na0, na1, nb0, nb1);
-            mfma_group(a0, a1, b0, b1, acc);
-            a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+            fetch(cur, kg + 1, na, nb);
+            group();
+            advance(na, nb);
         }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();  // every read of buffer `cur` has returned, slice kt + 1 is complete in the other one
-        if (HOT || kt + 1 < n_full_steps) fetch(cur ^ 1, 0, na0, na1, nb0, nb1);
+        if (HOT || kt + 1 < n_full_steps) fetch(cur ^ 1, 0, na, nb);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_group(a0, a1, b0, b1, acc);
-        a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+        group();
+        advance(na, nb);
     };
-    int kt = 0;
-    for (; kt + 2 < nk_full; ++kt) step(kt, std::true_type{});
-    for (; kt < n_full_steps; ++kt) step(kt, std::false_type{});
-    if (n_full_steps < nk) {
-        const int cur = n_full_steps & 1;
-        mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc,
-                       (g.K - n_full_steps * GEMM_BK + 7) / 8);
-        __syncthreads();
-    }
+    auto sweep = [&]() {
+        int kt = 0;
+        for (; kt + 2 < nk_full; ++kt) step(kt, std::true_type{});
+        for (; kt < n_full_steps; ++kt) step(kt, std::false_type{});
+        if (n_full_steps < nk) {
+            // Trailing partial slice: only the groups of 8 columns that hold data (the rest is zero).
+            const int cur = n_full_steps & 1;
+            const int kg_live = (g.K - n_full_steps * GEMM_BK + 7) / 8;
+            for (int kg = 0; kg < kg_live; ++kg) {
+                fetch(cur, kg, fa, fb);
+                group();
+            }
+            __syncthreads();
+        }
+    };
+    sweep();
 }
 
-constexpr int GEMM_LDS_FLOATS = 2 * (GEMM_TM + GEMM_TN) * GEMM_LDS_STRIDE;
+constexpr int GEMM_LDS_FLOATS = GemmSmall::LDS_FLOATS;
 
 inline bool gemm_operands_vectorizable(const GemmOperands& g) {
     return (reinterpret_cast<uintptr_t>(g.A) % 16 == 0) && (reinterpret_cast<uintptr_t>(g.B) % 16 == 0) &&

@@ -7,8 +7,8 @@
 
 namespace skm {
 
-// The double-buffered operand stages need 72 KiB of LDS, above the 64 KiB a kernel may use without
-// opting in; gfx950 has 160 KiB per CU, so two workgroups still fit on one CU.
+// The double-buffered operand stages need 72 KiB (small shape) or 144 KiB (large shape) of LDS, above the
+// 64 KiB a kernel may use without opting in; gfx950 has 160 KiB per CU.
 template <class Kernel>
 static int allow_large_lds(Kernel kernel, size_t bytes) {
     return check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -24,35 +24,52 @@ static int allow_large_lds(Kernel kernel, size_t bytes) {
         hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, __VA_ARGS__);                   \
     } while (0)
 
+// The large shape pays off once its tiles fill the chip a few times over; below that (hierarchical fine
+// clusterings, tests) the small shape wastes less on partial tiles and keeps more workgroups in flight.
+static bool use_big_tiles(int M, int N) {
+    if (M < 192 || N < 192) return false;
+    const long long tiles = (long long) ((M + GemmBig::TM - 1) / GemmBig::TM) * ((N + GemmBig::TN - 1) / GemmBig::TN);
+    return tiles >= 1024;
+}
+
+template <class S>
+static int fill_operands(GemmOperands& g, const float* A, int M, int64_t lda, const float* B, int N, int64_t ldb, int K) {
+    g.A = A; g.B = B; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
+    g.tiles_m = (M + S::TM - 1) / S::TM;
+    g.tiles_n = (N + S::TN - 1) / S::TN;
+    if ((long long) g.tiles_m * g.tiles_n > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
+    return SKM_OK;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Dense store: out[m][n] = D[m][n]                        (rotation, reference adsampling.h:191-215)
 //           or out[m][n] = -2 D[m][n] + rn[m] + cn[n]     (batch_computers.h:361-366)
 // Rows of D are the M operand (points), so that the 32 lanes of an accumulator column group write
 // 128 contiguous bytes of one output row.
 // ---------------------------------------------------------------------------------------------
-template <bool VEC, bool DIST>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_store_kernel(
+template <bool VEC, bool DIST, class S>
+__global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_store_kernel(
     GemmOperands g, float* __restrict__ out, int64_t ldo, const float* __restrict__ rn,
     const float* __restrict__ cn
 ) {
     extern __shared__ float lds[];
     int tm, tn;
     tile_of_block(g, blockIdx.x, tm, tn);
-    WaveAcc acc;
-    gemm_tile<VEC>(g, tm, tn, lds, acc);
+    WaveAccT<S::FM, S::FN> acc;
+    gemm_tile<VEC, S>(g, tm, tn, lds, acc);
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int m0 = tm * GEMM_TM + (wave >> 1) * 64;
-    const int n0 = tn * GEMM_TN + (wave & 1) * 64;
+    const int m0 = tm * S::TM + (wave / S::WN) * S::WAVE_M;
+    const int n0 = tn * S::TN + (wave % S::WN) * S::WAVE_N;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < S::FN; ++nb) {
         const int n = n0 + acc_col(nb, lane);
         if (n >= g.N) continue;
         float cnv = 0.0f;
         if (DIST) cnv = cn[n];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < S::FM; ++mb) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + acc_row(mb, r, lane);
@@ -66,83 +83,96 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_store_kernel(
     }
 }
 
+template <class S>
+static int launch_gemm_store_shape(skm_ctx* ctx, const float* A, int M, int64_t lda, const float* B, int N,
+                                   int64_t ldb, int K, float* out, int64_t ldo, const float* row_norm,
+                                   const float* col_norm) {
+    GemmOperands g;
+    SKM_TRY(fill_operands<S>(g, A, M, lda, B, N, ldb, K));
+    const bool vec = gemm_operands_vectorizable(g);
+    const bool dist = row_norm != nullptr && col_norm != nullptr;
+    const size_t lds_bytes = S::LDS_FLOATS * sizeof(float);
+    dim3 grid((unsigned) (g.tiles_m * g.tiles_n)), block(S::THREADS);
+    if (vec && dist)
+        SKM_LAUNCH_GEMM((gemm_store_kernel<true, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+    else if (vec)
+        SKM_LAUNCH_GEMM((gemm_store_kernel<true, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+    else if (dist)
+        SKM_LAUNCH_GEMM((gemm_store_kernel<false, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+    else
+        SKM_LAUNCH_GEMM((gemm_store_kernel<false, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+    return check_hip(hipGetLastError(), "gemm_store_kernel launch");
+}
+
 int launch_gemm_store(skm_ctx* ctx, const float* A, int M, int64_t lda, const float* B, int N,
                       int64_t ldb, int K, float* out, int64_t ldo, const float* row_norm,
                       const float* col_norm) {
     if (M <= 0 || N <= 0 || K <= 0) return SKM_OK;
-    GemmOperands g;
-    g.A = A; g.B = B; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
-    g.tiles_m = (M + GEMM_TM - 1) / GEMM_TM;
-    g.tiles_n = (N + GEMM_TN - 1) / GEMM_TN;
-    const long long total = (long long) g.tiles_m * g.tiles_n;
-    if (total > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
-    const bool vec = gemm_operands_vectorizable(g);
-    const bool dist = row_norm != nullptr && col_norm != nullptr;
-    const size_t lds_bytes = GEMM_LDS_FLOATS * sizeof(float);
-    dim3 grid((unsigned) total), block(GEMM_THREADS);
-    if (vec && dist)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<true, true>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
-    else if (vec)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<true, false>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
-    else if (dist)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<false, true>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
-    else
-        SKM_LAUNCH_GEMM((gemm_store_kernel<false, false>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
-    return check_hip(hipGetLastError(), "gemm_store_kernel launch");
+    if (use_big_tiles(M, N))
+        return launch_gemm_store_shape<GemmBig>(ctx, A, M, lda, B, N, ldb, K, out, ldo, row_norm, col_norm);
+    return launch_gemm_store_shape<GemmSmall>(ctx, A, M, lda, B, N, ldb, K, out, ldo, row_norm, col_norm);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Distance + argmin: the M operand is the centroid tile, the N operand the point tile, so every
-// lane owns one point column and scans 2 x 16 centroid rows in ascending index order in registers.
-// The two half-wavefronts (rows 0-3 | 4-7 of every group of 8) are merged with one cross-lane
-// exchange; the result of the 64-centroid granule is stored, never reduced with atomics.
+// lane owns one point column per accumulator block and scans its FM x 16 centroid rows in ascending
+// index order in registers.  The two half-wavefronts (rows 0-3 | 4-7 of every group of 8) are merged
+// with one cross-lane exchange; the result of the wavefront's granule (64 or 128 centroids, by shape)
+// is stored, never reduced with atomics.  The centroid norms of the tile go through LDS once the
+// operand stages are no longer read.
 // ---------------------------------------------------------------------------------------------
-template <bool VEC>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_argmin_kernel(
+template <bool VEC, class S>
+__global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_argmin_kernel(
     GemmOperands g, const float* __restrict__ xnorm, const float* __restrict__ cnorm,
     uint2* __restrict__ granule_min
 ) {
     extern __shared__ float lds[];
     int tm, tn;
     tile_of_block(g, blockIdx.x, tm, tn);
-    WaveAcc acc;
-    gemm_tile<VEC>(g, tm, tn, lds, acc);
+    float cn_mine = 0.0f;
+    if (threadIdx.x < S::TM) {
+        const int m = tm * S::TM + (int) threadIdx.x;
+        cn_mine = (m < g.M) ? cnorm[m] : 0.0f;
+    }
+    WaveAccT<S::FM, S::FN> acc;
+    gemm_tile<VEC, S>(g, tm, tn, lds, acc);
+    // Past the last barrier of the tile loop no wavefront reads the operand stages any more.
+    if (threadIdx.x < S::TM) lds[threadIdx.x] = cn_mine;
+    __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = tm * GEMM_TM + wm * 64;
-    const int n0 = tn * GEMM_TN + wn * 64;
-    const int granule = tm * 2 + wm;
+    const int wm = wave / S::WN, wn = wave % S::WN;
+    const int m0 = tm * S::TM + wm * S::WAVE_M;
+    const int n0 = tn * S::TN + wn * S::WAVE_N;
+    const int granule = tm * S::WM + wm;
     if (m0 >= g.M) return;  // granule entirely past the last centroid: never read by the merge
-
-    // ||c||^2 of the 32 rows this lane touches.
-    float cn[2][16];
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + acc_row(mb, r, lane);
-            cn[mb][r] = (m < g.M) ? cnorm[m] : 0.0f;
-        }
+    const float* cns = lds + wm * S::WAVE_M;
+    const bool whole = m0 + S::WAVE_M <= g.M;  // every row of the granule is a centroid
 
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < S::FN; ++nb) {
         const int n = n0 + acc_col(nb, lane);
         const float xn = (n < g.N) ? xnorm[n] : 0.0f;
+        // Row m0 + 4 * (lane / 32) may lie past M in the last granule; `have` says whether `best` is a centroid yet.
         float best = FLT_MAX;
         uint32_t best_idx = (uint32_t) m0;
         bool have = false;
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < S::FM; ++mb) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + acc_row(mb, r, lane);
-                const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn) + cn[mb][r];
-                if (m < g.M && (!have || v < best)) {
-                    best = v;
-                    best_idx = (uint32_t) m;
-                    have = true;
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const floatx4 c4 = *reinterpret_cast<const floatx4*>(&cns[acc_row(mb, r4 * 4, lane)]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int r = r4 * 4 + j;
+                    const int m = m0 + acc_row(mb, r, lane);
+                    const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn) + c4[j];
+                    if ((whole || m < g.M) && (!have || v < best)) {
+                        best = v;
+                        best_idx = (uint32_t) m;
+                        have = true;
+                    }
                 }
             }
         }
@@ -160,23 +190,34 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_argmin_kernel(
     }
 }
 
+template <class S>
+static int launch_gemm_argmin_shape(skm_ctx* ctx, const float* C, int k, const float* X, int n, int d,
+                                    int64_t ldc, int64_t ldx, const float* xnorm, const float* cnorm,
+                                    uint2* granule_min) {
+    GemmOperands g;
+    SKM_TRY(fill_operands<S>(g, C, k, ldc, X, n, ldx, d));
+    const size_t lds_bytes = S::LDS_FLOATS * sizeof(float);
+    dim3 grid((unsigned) (g.tiles_m * g.tiles_n)), block(S::THREADS);
+    if (gemm_operands_vectorizable(g))
+        SKM_LAUNCH_GEMM((gemm_argmin_kernel<true, S>), grid, block, lds_bytes, ctx->stream, g, xnorm, cnorm, granule_min);
+    else
+        SKM_LAUNCH_GEMM((gemm_argmin_kernel<false, S>), grid, block, lds_bytes, ctx->stream, g, xnorm, cnorm, granule_min);
+    return check_hip(hipGetLastError(), "gemm_argmin_kernel launch");
+}
+
+int gemm_argmin_granule(int k, int n) {
+    return use_big_tiles(k, n) ? GemmBig::WAVE_M : GemmSmall::WAVE_M;
+}
+
 int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int n, int d,
                        int64_t ldc, int64_t ldx, const float* xnorm, const float* cnorm,
-                       uint2* granule_min) {
+                       uint2* granule_min, int granule) {
     if (k <= 0 || n <= 0 || d <= 0) return SKM_OK;
-    GemmOperands g;
-    g.A = C; g.B = X; g.M = k; g.N = n; g.K = d; g.lda = ldc; g.ldb = ldx;
-    g.tiles_m = (k + GEMM_TM - 1) / GEMM_TM;
-    g.tiles_n = (n + GEMM_TN - 1) / GEMM_TN;
-    const long long total = (long long) g.tiles_m * g.tiles_n;
-    if (total > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
-    const size_t lds_bytes = GEMM_LDS_FLOATS * sizeof(float);
-    dim3 grid((unsigned) total), block(GEMM_THREADS);
-    if (gemm_operands_vectorizable(g))
-        SKM_LAUNCH_GEMM((gemm_argmin_kernel<true>), grid, block, lds_bytes, ctx->stream, g, xnorm, cnorm, granule_min);
-    else
-        SKM_LAUNCH_GEMM((gemm_argmin_kernel<false>), grid, block, lds_bytes, ctx->stream, g, xnorm, cnorm, granule_min);
-    return check_hip(hipGetLastError(), "gemm_argmin_kernel launch");
+    if (granule == GemmBig::WAVE_M)
+        return launch_gemm_argmin_shape<GemmBig>(ctx, C, k, X, n, d, ldc, ldx, xnorm, cnorm, granule_min);
+    if (granule == GemmSmall::WAVE_M)
+        return launch_gemm_argmin_shape<GemmSmall>(ctx, C, k, X, n, d, ldc, ldx, xnorm, cnorm, granule_min);
+    return set_error(SKM_ERR_INVALID, "unsupported argmin granule");
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -419,13 +460,13 @@ int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, 
 //       m = first minimum of the batch;  if (m < out) { out = max(0, m); idx = argmin; }
 // ---------------------------------------------------------------------------------------------
 __global__ void merge_granules_kernel(
-    const uint2* __restrict__ granule_min, int n, int k, uint32_t* __restrict__ out_idx,
+    const uint2* __restrict__ granule_min, int n, int k, int granule, uint32_t* __restrict__ out_idx,
     float* __restrict__ out_dist
 ) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    const int n_granules = (k + 63) / 64;
-    const int per_batch = SKM_Y_BATCH_SIZE / 64;
+    const int n_granules = (k + granule - 1) / granule;
+    const int per_batch = SKM_Y_BATCH_SIZE / granule;
     float out = FLT_MAX;
     uint32_t idx = 0;
     for (int g0 = 0; g0 < n_granules; g0 += per_batch) {
@@ -449,11 +490,11 @@ __global__ void merge_granules_kernel(
     out_dist[i] = out;
 }
 
-int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, uint32_t* out_idx,
+int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, int granule, uint32_t* out_idx,
                           float* out_dist) {
     if (n <= 0) return SKM_OK;
     dim3 grid((n + 255) / 256), block(256);
-    hipLaunchKernelGGL(merge_granules_kernel, grid, block, 0, ctx->stream, granule_min, n, k, out_idx, out_dist);
+    hipLaunchKernelGGL(merge_granules_kernel, grid, block, 0, ctx->stream, granule_min, n, k, granule, out_idx, out_dist);
     return check_hip(hipGetLastError(), "merge_granules_kernel launch");
 }
 

@@ -84,13 +84,15 @@ int launch_gemm_store(skm_ctx* ctx, const float* A, int M, int64_t lda, const fl
                       int64_t ldb, int K, float* out, int64_t ldo, const float* row_norm,
                       const float* col_norm);
 
-// Per (granule of 64 centroids, point) minimum of -2 x.c + |x|^2 + |c|^2 and its lowest index,
-// written as uint2 {float bits, index} to granule_min[granule * n + point].
+// Per (granule of consecutive centroids, point) minimum of -2 x.c + |x|^2 + |c|^2 and its lowest index,
+// written as uint2 {float bits, index} to granule_min[granule * n + point].  The granule size (64 or 128,
+// a divisor of the 1024-centroid batch) follows from the tile shape picked for the problem size.
+int gemm_argmin_granule(int k, int n);
 int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int n, int d,
                        int64_t ldc, int64_t ldx, const float* xnorm, const float* cnorm,
-                       uint2* granule_min);
+                       uint2* granule_min, int granule);
 
-int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, uint32_t* out_idx,
+int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, int granule, uint32_t* out_idx,
                           float* out_dist);
 
 // Number of striped copies of the per-stage accounting counters (each n_hblocks + 2 entries long).

@@ -117,7 +117,7 @@ int skm_assign_full(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, 
     SKM_REQUIRE(k > 0 && d > 0, "k and d must be positive");
     SKM_REQUIRE(k <= 0x7fffffffULL && d <= (1u << 20), "k or d out of range");
     ScopedStage outer(ctx, "search");
-    const size_t n_granules = (k + 63) / 64;
+    const size_t n_granules = (k + 63) / 64;  // the smallest granule: an upper bound for every chunk
     // Points per chunk so that the granule scratch respects the workspace limit.
     size_t chunk = ctx->workspace_limit / (n_granules * sizeof(uint2));
     chunk = std::max<size_t>(128, (chunk / 128) * 128);
@@ -127,14 +127,15 @@ int skm_assign_full(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, 
     SKM_TRY(workspace(ctx, 0, n_granules * std::min(chunk, n) * sizeof(uint2), &scratch));
     for (size_t i0 = 0; i0 < n; i0 += chunk) {
         const size_t m = std::min(chunk, n - i0);
+        const int granule = gemm_argmin_granule((int) k, (int) m);
         {
             ScopedStage st(ctx, "search/1st_blas");
             SKM_TRY(launch_gemm_argmin(ctx, d_c, (int) k, d_x + i0 * d, (int) m, (int) d, (int64_t) d, (int64_t) d,
-                                       d_xnorm + i0, d_cnorm, (uint2*) scratch));
+                                       d_xnorm + i0, d_cnorm, (uint2*) scratch, granule));
         }
         {
             ScopedStage st(ctx, "search/merge");
-            SKM_TRY(launch_merge_granules(ctx, (const uint2*) scratch, (int) m, (int) k, d_out_idx + i0,
+            SKM_TRY(launch_merge_granules(ctx, (const uint2*) scratch, (int) m, (int) k, granule, d_out_idx + i0,
                                           d_out_dist + i0));
         }
     }
