@@ -233,11 +233,20 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
 //   * a point's candidates are appended batch after batch (a batch of 1024 centroids = 8 consecutive
 //     tiles), which lets the pruning kernel walk its list once;
 //   * ||x||^2 and the thresholds of the workgroup's points stay in registers for the whole sweep, the
-//     128 centroid norms of a tile are staged through LDS: the epilogue issues no global load;
-//   * the first operand slice of tile t+1 is requested during the last MFMA step of tile t and lands
-//     while the epilogue of tile t runs, so neither the prologue nor the epilogue latency is exposed.
+//     128 centroid norms of a tile are staged through LDS: the epilogue issues no global load.
+// d' is short (16 to a few hundred columns), so a tile is only one to a few operand slices long and a
+// per-tile prologue would cost as much as the tile.  The slices of all tiles therefore form ONE software
+// pipeline: while slice s is multiplied, slice s + 1 sits in the other LDS buffer and slice s + 2 is on
+// its way into registers, across tile boundaries; a tile's epilogue runs after the last group of its
+// last slice with the loads of the next tiles in flight.  Step s (LDS buffer s & 1):
+//   registers (slice s + 1) -> other buffer; request slice s + 2; groups of 8 columns with the next
+//   group's fragments fetched ahead; workgroup barrier before the last group; first fragments of slice
+//   s + 1; last group; epilogue if the tile ends here.
+// FAST: rows are 16-byte aligned and hold at least round_up(d', 32) columns, so every slice is fetched
+// without guards; columns at or past d' in the last group are zeroed in the centroid fragments (finite
+// point values times zero add nothing).  Otherwise slices are fetched with guards (zeros past d').
 // Workgroups of one XCD sweep the centroid tiles roughly in step and share them through that XCD's L2.
-template <bool VEC>
+template <bool FAST>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     GemmOperands g, const float* __restrict__ xnorm, const float* __restrict__ cnorm,
     const float* __restrict__ thr0, uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap
@@ -245,9 +254,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     extern __shared__ float lds[];
     float* As = lds;
     float* Bs = lds + 2 * GEMM_TM * GEMM_LDS_STRIDE;
-    float* cn_s = lds + GEMM_LDS_FLOATS;  // [2][GEMM_TM]
+    float* cn_s = lds + GEMM_LDS_FLOATS;  // [3][GEMM_TM]: tile t uses slot t % 3 (written two tiles ahead of its readers' successors)
     // The workgroup is the only writer of its points' lists, so the slot counters live in LDS.
-    uint32_t* cnt_s = reinterpret_cast<uint32_t*>(cn_s + 2 * GEMM_TM);  // [GEMM_TN]
+    uint32_t* cnt_s = reinterpret_cast<uint32_t*>(cn_s + 3 * GEMM_TM);  // [GEMM_TN]
     const int tn = blockIdx.x;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -256,7 +265,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     const int ld_row = tid >> 3;
     const int ld_k = (tid & 7) * 4;
 
-    // Row offsets of the four point rows this thread stages (clamped: padding points never pass).
+    // Rows of the four point rows this thread stages (clamped: padding points never pass).
     const float* b_rows[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
@@ -267,57 +276,48 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     // The two points of this lane.
     int pt[2];
     float xn[2], thr[2];
+    uint2* list[2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
         pt[nb] = tn * GEMM_TN + wn * 64 + acc_col(nb, lane);
         const bool valid = pt[nb] < g.N;
         xn[nb] = valid ? xnorm[pt[nb]] : 0.0f;
         thr[nb] = valid ? thr0[pt[nb]] : -3.0e38f;  // nothing passes for padding columns
+        list[nb] = cand + (int64_t) (valid ? pt[nb] : 0) * cap;
     }
 
-    uint2* list[2];
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) list[nb] = cand + (int64_t) (pt[nb] < g.N ? pt[nb] : 0) * cap;
-
-    const int nk_full = VEC ? g.K / GEMM_BK : 0;       // slices fetched without guards
-    const int n_full_steps = g.K / GEMM_BK;            // slices whose 32 columns all hold data
-    const bool has_tail = (g.K % GEMM_BK) != 0;
-    const int tail_groups = (g.K % GEMM_BK + 7) / 8;
+    const int nk = (g.K + GEMM_BK - 1) / GEMM_BK;              // slices per tile
+    const int last_groups = (g.K - (nk - 1) * GEMM_BK + 7) / 8;  // groups of 8 columns in a tile's last slice
+    const int total = g.tiles_m * nk;                           // slices of the whole sweep
+    // FAST: columns of the last group at or past d' (this lane supplies columns 4 * (lane / 32) + i of a group).
+    const int last_col0 = (nk - 1) * GEMM_BK + (last_groups - 1) * 8 + (lane >> 5) * 4;
     floatx4 ra[4], rb[4];
     float cn_next = 0.0f;
 
-    // Operand slice `kt` of centroid tile `tm`, every column in range (no guard, loads issued back to back).
-    auto request_full = [&](int tm, int kt) {
+    // Slice (tm, kt) -> registers, together with one centroid norm of that tile per thread.  Every load is
+    // unconditional (a load under a condition would have to be waited for right where it is issued).
+    auto request = [&](int tm, int kt) {
         const int k0 = kt * GEMM_BK;
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             int r = tm * GEMM_TM + ld_row + 32 * p;
             r = r < g.M ? r : g.M - 1;
-            ra[p] = load_k4<VEC, false>(g.A + (int64_t) r * g.lda + ld_k, k0, g.K);
-            rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            const float* a_row = g.A + (int64_t) r * g.lda;
+            if (FAST) {
+                ra[p] = load_k4<true, false>(a_row + ld_k, k0, g.K);
+                rb[p] = load_k4<true, false>(b_rows[p], k0, g.K);
+            } else {
+                ra[p] = load_k4<false, true>(a_row, k0 + ld_k, g.K);
+                rb[p] = load_k4<false, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
+            }
         }
-    };
-    // Same with columns at or past K read as zero (trailing slice; every slice of the scalar path).
-    auto request_guarded = [&](int tm, int kt) {
-        const int k0 = kt * GEMM_BK + ld_k;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            int r = tm * GEMM_TM + ld_row + 32 * p;
-            r = r < g.M ? r : g.M - 1;
-            ra[p] = load_k4<VEC, true>(g.A + (int64_t) r * g.lda, k0, g.K);
-            rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0, g.K);
-        }
-    };
-    // First slice of tile `tm` plus that tile's centroid norms (rows past M get a norm nothing passes with).
-    auto request_first = [&](int tm) {
-        if (nk_full > 0) request_full(tm, 0); else request_guarded(tm, 0);
-        if (tid < GEMM_TM) {
-            const int m = tm * GEMM_TM + tid;
-            cn_next = m < g.M ? cnorm[m] : 3.0e38f;
-        }
+        const int m = tm * GEMM_TM + (tid & (GEMM_TM - 1));
+        cn_next = cnorm[m < g.M ? m : g.M - 1];
     };
     const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
-    auto publish = [&](int buf) {
+    // Registers -> LDS buffer `buf`; `first_of` >= 0: the slice opens tile `first_of`, whose norms go along
+    // (rows past M get a norm nothing passes with).
+    auto publish = [&](int buf, int first_of) {
         float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + st_off;
         float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + st_off;
 #pragma unroll
@@ -325,82 +325,43 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
             *reinterpret_cast<floatx4*>(&as[32 * p * GEMM_LDS_STRIDE]) = ra[p];
             *reinterpret_cast<floatx4*>(&bs[32 * p * GEMM_LDS_STRIDE]) = rb[p];
         }
+        if (first_of >= 0 && tid < GEMM_TM)
+            cn_s[(first_of % 3) * GEMM_TM + tid] = (first_of * GEMM_TM + tid < g.M) ? cn_next : 3.0e38f;
     };
-
-    int cur = 0;
-    request_first(0);
-    publish(0);
-    if (tid < GEMM_TM) {
-        cn_s[tid] = cn_next;
-        cnt_s[tid] = 0u;
-    }
-    __syncthreads();
-
     const int frag_off = (lane & 31) * GEMM_LDS_STRIDE + (lane >> 5) * 4;
     const int a_frag = (wm * 64) * GEMM_LDS_STRIDE + frag_off;
     const int b_frag = (wn * 64) * GEMM_LDS_STRIDE + frag_off;
-    for (int tm = 0; tm < g.tiles_m; ++tm) {
-        WaveAcc acc;
+    auto fetch = [&](int buf, int kg, floatx4& f0, floatx4& f1, floatx4& g0, floatx4& g1) {
+        const float* as = As + buf * GEMM_TM * GEMM_LDS_STRIDE + a_frag + kg * 8;
+        const float* bs = Bs + buf * GEMM_TN * GEMM_LDS_STRIDE + b_frag + kg * 8;
+        f0 = *reinterpret_cast<const floatx4*>(as);
+        f1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
+        g0 = *reinterpret_cast<const floatx4*>(bs);
+        g1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
+    };
+
+    WaveAcc acc;
+    auto clear = [&]() {
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc.v[mb][nb][r] = 0.0f;
-        const bool next_tile = (tm + 1) < g.tiles_m;
+    };
 
-        // Full slices whose successor is a full slice of the same tile: the hot loop, free of guards.
-        for (int kt = 0; kt + 1 < nk_full; ++kt) {
-            request_full(tm, kt + 1);
-            __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the MFMAs they overlap with
-            mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
-            __builtin_amdgcn_sched_barrier(0);
-            publish(cur ^ 1);
-            __syncthreads();
-            cur ^= 1;
-        }
-        // Scalar path: every slice is fetched with guards.
-        if (!VEC) {
-            for (int kt = 0; kt + 1 < n_full_steps; ++kt) {
-                request_guarded(tm, kt + 1);
-                mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
-                publish(cur ^ 1);
-                __syncthreads();
-                cur ^= 1;
-            }
-        }
-        // Last full slice: its successor is the trailing partial slice or the next tile's first slice.
-        if (n_full_steps > 0) {
-            if (has_tail) {
-                request_guarded(tm, n_full_steps);
-            } else if (next_tile) {
-                request_first(tm + 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_step_full(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc);
-            if (has_tail) {
-                publish(cur ^ 1);
-                __syncthreads();
-                cur ^= 1;
-            }
-        }
-        if (has_tail) {
-            if (next_tile) request_first(tm + 1);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_step_tail(As + cur * GEMM_TM * GEMM_LDS_STRIDE + a_frag, Bs + cur * GEMM_TN * GEMM_LDS_STRIDE + b_frag, acc, tail_groups);
-        }
-
-        // ---- epilogue of tile tm: first pruning test, candidates appended to the per-point lists ----
-        const float* cns = cn_s + (tm & 1) * GEMM_TM + wm * 64;
+    // First pruning test of tile tm and the appends to the per-point lists.  Passing pairs are rare (a fraction
+    // of a percent).  The outcome of the 32 tests of one point is collected in a per-lane bit mask (the sign of
+    // v - thr is shifted in, so a test costs four vector instructions and no scalar dependency); lanes with an
+    // empty mask skip the append.
+    auto epilogue = [&](int tm) {
+        const float* cns = cn_s + (tm % 3) * GEMM_TM + wm * 64;
         const int m0 = tm * GEMM_TM + wm * 64;
-        // Passing pairs are rare (a fraction of a percent).  The outcome of the 32 tests of one point is
-        // collected in a per-lane bit mask (the sign of v - thr is shifted in, so a test costs four vector
-        // instructions and no scalar dependency); lanes with an empty mask skip the append.
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
             uint32_t pass = 0;  // element (mb, r) lands in bit 31 - (mb * 16 + r)
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+            for (int mb = 0; mb < 2; ++mb) {
 #pragma unroll
                 for (int r4 = 0; r4 < 4; ++r4) {
                     const floatx4 c4 = *reinterpret_cast<const floatx4*>(&cns[acc_row(mb, r4 * 4, lane)]);
@@ -413,6 +374,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
                         pass = __builtin_amdgcn_alignbit(pass, __float_as_uint(v - thr[nb]), 31);
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);  // bounds how many norms are held at once
+            }
             if (pass) {
                 uint32_t slot = atomicAdd(&cnt_s[wn * 64 + acc_col(nb, lane)], (uint32_t) __popc(pass));
 #pragma unroll
@@ -427,13 +390,73 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
                     }
             }
         }
-        if (next_tile) {
-            publish(cur ^ 1);
-            if (tid < GEMM_TM) cn_s[((tm + 1) & 1) * GEMM_TM + tid] = cn_next;
+    };
+
+    // Prologue: slice 0 in buffer 0, slice 1 in registers, first fragments of slice 0 fetched.  The request
+    // cursor stops at the last slice: requests past the end fetch that slice again and are never published.
+    int req_tm = 0, req_kt = 0;
+    auto advance_cursor = [&]() {
+        if (req_kt + 1 < nk) {
+            ++req_kt;
+        } else if (req_tm + 1 < g.tiles_m) {
+            req_kt = 0;
+            ++req_tm;
         }
-        __syncthreads();
-        cur ^= 1;
+    };
+    if (tid < GEMM_TN) cnt_s[tid] = 0u;
+    request(0, 0);
+    advance_cursor();
+    publish(0, 0);
+    int pub_tm = req_tm, pub_kt = req_kt;  // slice held in the registers (next to publish)
+    request(req_tm, req_kt);
+    advance_cursor();
+    __syncthreads();
+    floatx4 a0, a1, b0, b1;
+    fetch(0, 0, a0, a1, b0, b1);
+    clear();
+
+    int s = 0;
+    for (int tm = 0; tm < g.tiles_m; ++tm) {
+        for (int kt = 0; kt < nk; ++kt, ++s) {
+            const int cur = s & 1;
+            const bool last = kt + 1 == nk;
+            if (s + 1 < total) publish(cur ^ 1, pub_kt == 0 ? pub_tm : -1);
+            pub_tm = req_tm;
+            pub_kt = req_kt;
+            request(req_tm, req_kt);
+            advance_cursor();
+            __builtin_amdgcn_sched_barrier(0);
+            // The accumulators flow through one straight line of code: a branch around MFMAs would make the
+            // register allocator keep two copies of them.
+            floatx4 na0, na1, nb0, nb1;
+            const int n_ahead = (last ? last_groups : GEMM_BK / 8) - 1;
+            for (int kg = 0; kg < n_ahead; ++kg) {
+                fetch(cur, kg + 1, na0, na1, nb0, nb1);
+                mfma_group(a0, a1, b0, b1, acc);
+                a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+            }
+            if (FAST) {
+                // zero the centroid columns at or past d' in the last group of the tile's last slice
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool live = !last || last_col0 + i < g.K;
+                    a0[i] = live ? a0[i] : 0.0f;
+                    a1[i] = live ? a1[i] : 0.0f;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();  // every read of buffer `cur` has returned, slice s + 1 is complete in the other one
+            fetch(cur ^ 1, 0, na0, na1, nb0, nb1);  // past the last slice: stale data, never used
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_group(a0, a1, b0, b1, acc);
+            a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
+            if (last) {
+                epilogue(tm);
+                clear();
+            }
+        }
     }
+    __syncthreads();
     if (tid < GEMM_TN && tn * GEMM_TN + tid < g.N) cand_count[tn * GEMM_TN + tid] = cnt_s[tid];
 }
 
@@ -442,12 +465,11 @@ int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, 
                            uint2* cand, uint32_t cap) {
     if (k <= 0 || n <= 0 || partial_d <= 0) return SKM_OK;
     GemmOperands g;
-    g.A = C; g.B = X; g.M = k; g.N = n; g.K = partial_d; g.lda = ld; g.ldb = ld;
-    g.tiles_m = (k + GEMM_TM - 1) / GEMM_TM;
-    g.tiles_n = (n + GEMM_TN - 1) / GEMM_TN;
-    const size_t lds_bytes = (GEMM_LDS_FLOATS + 2 * GEMM_TM + GEMM_TN) * sizeof(float);
+    SKM_TRY(fill_operands<GemmSmall>(g, C, k, ld, X, n, ld, partial_d));
+    const size_t lds_bytes = (GEMM_LDS_FLOATS + 3 * GEMM_TM + GEMM_TN) * sizeof(float);
     dim3 grid((unsigned) g.tiles_n), block(GEMM_THREADS);
-    if (gemm_operands_vectorizable(g))
+    const int64_t padded_k = ((int64_t) partial_d + GEMM_BK - 1) / GEMM_BK * GEMM_BK;
+    if (gemm_operands_vectorizable(g) && padded_k <= ld)
         SKM_LAUNCH_GEMM((gemm_candidates_kernel<true>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
     else
         SKM_LAUNCH_GEMM((gemm_candidates_kernel<false>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
