@@ -46,6 +46,7 @@ struct GemmShape {
     static constexpr int NLA = TM / ROWS_PER_LOAD;     // loads per thread and slice, A operand
     static constexpr int NLB = TN / ROWS_PER_LOAD;
     static constexpr int LDS_FLOATS = 2 * (TM + TN) * GEMM_LDS_STRIDE;
+    static constexpr int BAND = WG_PER_CU == 1 ? 4 : 8;  // M-tiles per band of the workgroup-to-tile map
     static_assert(TM % ROWS_PER_LOAD == 0 && TN % ROWS_PER_LOAD == 0, "tile rows must split evenly over the loads");
 };
 using GemmSmall = GemmShape<2, 2, 2, 2, 2>;
@@ -82,18 +83,20 @@ __device__ __forceinline__ int acc_col(int nb, int lane) {
 
 // Maps the hardware workgroup id to a tile so that the workgroups resident on
 // one XCD (ids congruent mod 8 are dispatched to the same XCD) cover a compact
-// block of 8 M-tiles x several N-tiles and share operand panels in that XCD's L2.
+// block of BAND M-tiles x several N-tiles and share operand panels in that XCD's L2
+// (64 resident workgroups of the small shape: 8 x 8; 32 of the large one: 4 x 8).
+template <int BAND>
 __device__ __forceinline__ void tile_of_block(const GemmOperands& g, int bid, int& tm, int& tn) {
     const int total = g.tiles_m * g.tiles_n;
     const int q = total / GEMM_XCDS, r = total % GEMM_XCDS;
     const int x = bid % GEMM_XCDS, within = bid / GEMM_XCDS;
     const int L = x * q + (x < r ? x : r) + within;
-    const int band_tiles = 8 * g.tiles_n;
+    const int band_tiles = BAND * g.tiles_n;
     const int band = L / band_tiles;
     const int in_band = L - band * band_tiles;
-    const int rows_in_band = (g.tiles_m - band * 8) < 8 ? (g.tiles_m - band * 8) : 8;
+    const int rows_in_band = (g.tiles_m - band * BAND) < BAND ? (g.tiles_m - band * BAND) : BAND;
     tn = in_band / rows_in_band;
-    tm = band * 8 + in_band % rows_in_band;
+    tm = band * BAND + in_band % rows_in_band;
 }
 
 // Four consecutive operand columns starting at k.  GUARD: columns at or past K read as zero (last,
@@ -119,6 +122,18 @@ __device__ __forceinline__ floatx4 load_k4(const float* row, int k, int K) {
         v.w = (k + 3 < K) ? row[k + 3] : 0.0f;
     }
     return v;
+}
+
+// 16 bytes through a buffer descriptor: address = descriptor base + voffset (per lane, bytes) + soffset
+// (wavefront-uniform, bytes).  One 32-bit register per lane addresses a row whatever the step, where a
+// pointer per load would take two.
+typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t operand_rows(const float* base) {
+    // raw buffer, no stride, no bounds clamp needed (rows are clamped by the caller); dword 3 = 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ floatx4 load_rows_x4(__amdgpu_buffer_rsrc_t rows, uint32_t voffset, uint32_t soffset) {
+    return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rows, (int) voffset, (int) soffset, 0));
 }
 
 // One full BK step of a wavefront's 64 x 64 quadrant: 4 groups of 8 columns, 16 MFMAs each; the
@@ -205,22 +220,26 @@ __device__ __forceinline__ void gemm_tile(
     const int wm = wave / S::WN, wn = wave % S::WN;
 
     // Global -> register staging: thread covers rows (tid / 8) + ROWS_PER_LOAD * p, 4 floats at column 4 * (tid % 8).
-    // Rows past the end are clamped to the last row: duplicates are masked by the epilogue.
+    // Rows past the end are clamped to the last row: duplicates are masked by the epilogue.  Unguarded slices
+    // are fetched through one buffer descriptor per operand (tile base, wavefront-uniform) plus a 32-bit byte
+    // offset per row; the slice's column offset is a scalar.
     const int ld_row = tid >> 3;
     const int ld_k = (tid & 7) * 4;
-    const float* a_rows[S::NLA];
-    const float* b_rows[S::NLB];
+    const float* a_base = g.A + (int64_t) (tm * S::TM) * g.lda;
+    const float* b_base = g.B + (int64_t) (tn * S::TN) * g.ldb;
+    const __amdgpu_buffer_rsrc_t a_desc = operand_rows(a_base);
+    const __amdgpu_buffer_rsrc_t b_desc = operand_rows(b_base);
+    uint32_t a_off[S::NLA], b_off[S::NLB];  // bytes from the tile base to this thread's 4 columns of slice 0
+    const int a_last = g.M - 1 - tm * S::TM, b_last = g.N - 1 - tn * S::TN;
 #pragma unroll
     for (int p = 0; p < S::NLA; ++p) {
-        int r = tm * S::TM + ld_row + S::ROWS_PER_LOAD * p;
-        r = r < g.M ? r : g.M - 1;
-        a_rows[p] = g.A + (int64_t) r * g.lda + ld_k;
+        const int r = ld_row + S::ROWS_PER_LOAD * p;
+        a_off[p] = ((uint32_t) (r < a_last ? r : a_last) * (uint32_t) g.lda + (uint32_t) ld_k) * 4u;
     }
 #pragma unroll
     for (int p = 0; p < S::NLB; ++p) {
-        int r = tn * S::TN + ld_row + S::ROWS_PER_LOAD * p;
-        r = r < g.N ? r : g.N - 1;
-        b_rows[p] = g.B + (int64_t) r * g.ldb + ld_k;
+        const int r = ld_row + S::ROWS_PER_LOAD * p;
+        b_off[p] = ((uint32_t) (r < b_last ? r : b_last) * (uint32_t) g.ldb + (uint32_t) ld_k) * 4u;
     }
     floatx4 ra[S::NLA], rb[S::NLB];
 
@@ -239,14 +258,14 @@ __device__ __forceinline__ void gemm_tile(
         const int k0 = kt * GEMM_BK;
         if (kt < nk_full) {
 #pragma unroll
-            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_rows_x4(a_desc, a_off[p], (uint32_t) k0 * 4u);
 #pragma unroll
-            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_rows_x4(b_desc, b_off[p], (uint32_t) k0 * 4u);
         } else {
 #pragma unroll
-            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, true>(a_rows[p] - ld_k, k0 + ld_k, g.K);
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, true>(a_base + (a_off[p] / 4u - ld_k), k0 + ld_k, g.K);
 #pragma unroll
-            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, true>(b_rows[p] - ld_k, k0 + ld_k, g.K);
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, true>(b_base + (b_off[p] / 4u - ld_k), k0 + ld_k, g.K);
         }
     };
     const int st_off = ld_row * GEMM_LDS_STRIDE + ld_k;
@@ -303,9 +322,9 @@ __device__ __forceinline__ void gemm_tile(
             publish(cur ^ 1);
             const int k0 = (kt + 2) * GEMM_BK;
 #pragma unroll
-            for (int p = 0; p < S::NLA; ++p) ra[p] = load_k4<VEC, false>(a_rows[p], k0, g.K);
+            for (int p = 0; p < S::NLA; ++p) ra[p] = load_rows_x4(a_desc, a_off[p], (uint32_t) k0 * 4u);
 #pragma unroll
-            for (int p = 0; p < S::NLB; ++p) rb[p] = load_k4<VEC, false>(b_rows[p], k0, g.K);
+            for (int p = 0; p < S::NLB; ++p) rb[p] = load_rows_x4(b_desc, b_off[p], (uint32_t) k0 * 4u);
         } else {
             if (kt + 1 < nk) publish(cur ^ 1);
             if (kt + 2 < nk) request(kt + 2);

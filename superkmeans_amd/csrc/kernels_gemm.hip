@@ -54,7 +54,7 @@ __global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_store_kernel(
 ) {
     extern __shared__ float lds[];
     int tm, tn;
-    tile_of_block(g, blockIdx.x, tm, tn);
+    tile_of_block<S::BAND>(g, blockIdx.x, tm, tn);
     WaveAccT<S::FM, S::FN> acc;
     gemm_tile<VEC, S>(g, tm, tn, lds, acc);
 
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_argmin_kernel(
 ) {
     extern __shared__ float lds[];
     int tm, tn;
-    tile_of_block(g, blockIdx.x, tm, tn);
+    tile_of_block<S::BAND>(g, blockIdx.x, tm, tn);
     float cn_mine = 0.0f;
     if (threadIdx.x < S::TM) {
         const int m = tm * S::TM + (int) threadIdx.x;
