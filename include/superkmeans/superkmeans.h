@@ -731,13 +731,19 @@ class SuperKMeans {
     }
 
     std::vector<centroid_value_t> GetOutputCentroids(bool should_unrotate) {
-        std::vector<centroid_value_t> out(n_clusters * d);
+        // With a sink set the centroids go straight to the caller's buffer and the returned vector is empty.
+        std::vector<centroid_value_t> out;
+        centroid_value_t* dst = output_sink;
+        if (dst == nullptr) {
+            out.resize(n_clusters * d);
+            dst = out.data();
+        }
         if (should_unrotate) {
             dbuf<float> unrotated(ctx, n_clusters * d);
             pruner->Unrotate(horizontal_centroids.get(), unrotated.get(), n_clusters);
-            unrotated.Download(out.data(), n_clusters * d);
+            unrotated.Download(dst, n_clusters * d);
         } else {
-            horizontal_centroids.Download(out.data(), n_clusters * d);
+            horizontal_centroids.Download(dst, n_clusters * d);
         }
         return out;
     }
@@ -853,6 +859,10 @@ class SuperKMeans {
   public:
     std::unique_ptr<uint32_t[]> assignments;
     std::vector<SuperKMeansIterationStats> iteration_stats;
+    // Not in the reference.  When set, Train() writes the n_clusters * d centroids here and returns an empty
+    // vector: the C ABI passes the caller's buffer in, which saves a zero-filled temporary and a copy (41 MB
+    // each at k=10,000, d=1024).
+    centroid_value_t* output_sink = nullptr;
 };
 
 } // namespace skmeans

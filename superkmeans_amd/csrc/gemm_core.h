@@ -136,52 +136,6 @@ __device__ __forceinline__ floatx4 load_rows_x4(__amdgpu_buffer_rsrc_t rows, uin
     return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(rows, (int) voffset, (int) soffset, 0));
 }
 
-// One full BK step of a wavefront's 64 x 64 quadrant: 4 groups of 8 columns, 16 MFMAs each; the
-// fragments of the next group are requested before the current group's MFMAs.
-__device__ __forceinline__ void mfma_step_full(const float* as, const float* bs, WaveAcc& acc) {
-    floatx4 a0 = *reinterpret_cast<const floatx4*>(as);
-    floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE);
-    floatx4 b0 = *reinterpret_cast<const floatx4*>(bs);
-    floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE);
-#pragma unroll
-    for (int kg = 0; kg < GEMM_BK / 8; ++kg) {
-        floatx4 na0, na1, nb0, nb1;
-        if (kg + 1 < GEMM_BK / 8) {
-            na0 = *reinterpret_cast<const floatx4*>(as + (kg + 1) * 8);
-            na1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
-            nb0 = *reinterpret_cast<const floatx4*>(bs + (kg + 1) * 8);
-            nb1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + (kg + 1) * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
-            acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
-            acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
-            acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
-        }
-        if (kg + 1 < GEMM_BK / 8) {
-            a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
-        }
-    }
-}
-
-// Trailing partial step: only the `kg_live` groups of 8 columns that hold data (the rest is zero).
-__device__ __forceinline__ void mfma_step_tail(const float* as, const float* bs, WaveAcc& acc, int kg_live) {
-    for (int kg = 0; kg < kg_live; ++kg) {
-        const floatx4 a0 = *reinterpret_cast<const floatx4*>(as + kg * 8);
-        const floatx4 a1 = *reinterpret_cast<const floatx4*>(as + 32 * GEMM_LDS_STRIDE + kg * 8);
-        const floatx4 b0 = *reinterpret_cast<const floatx4*>(bs + kg * 8);
-        const floatx4 b1 = *reinterpret_cast<const floatx4*>(bs + 32 * GEMM_LDS_STRIDE + kg * 8);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b0[i], acc.v[0][0], 0, 0, 0);
-            acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[i], b1[i], acc.v[0][1], 0, 0, 0);
-            acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b0[i], acc.v[1][0], 0, 0, 0);
-            acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[i], b1[i], acc.v[1][1], 0, 0, 0);
-        }
-    }
-}
-
 // The 16 MFMAs of one group of 8 columns (fragments a0, a1, b0, b1 hold 4 columns each per lane).
 __device__ __forceinline__ void mfma_group(const floatx4& a0, const floatx4& a1, const floatx4& b0, const floatx4& b1,
                                            WaveAcc& acc) {

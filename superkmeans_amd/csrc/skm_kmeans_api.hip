@@ -132,8 +132,8 @@ int skm_kmeans_train(skm_kmeans* km, const float* h_data, size_t n, const float*
                      float* h_out_centroids) {
     if (!km || !h_data || !h_out_centroids) return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_train: null argument");
     SKM_API_GUARD({
-        auto c = km->hier ? km->hier->Train(h_data, n, h_queries, n_queries) : km->flat->Train(h_data, n, h_queries, n_queries);
-        std::memcpy(h_out_centroids, c.data(), c.size() * sizeof(float));
+        km->base()->output_sink = h_out_centroids;  // centroids are downloaded straight into the caller's buffer
+        if (km->hier) km->hier->Train(h_data, n, h_queries, n_queries); else km->flat->Train(h_data, n, h_queries, n_queries);
         km->n_trained = n;
     });
 }
@@ -143,9 +143,9 @@ int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, const
     if (!km || !d_data || !h_out_centroids)
         return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_train_device: null argument");
     SKM_API_GUARD({
-        auto c = km->hier ? km->hier->TrainDevice(d_data, n, d_queries, n_queries)
-                          : km->flat->TrainDevice(d_data, n, d_queries, n_queries);
-        std::memcpy(h_out_centroids, c.data(), c.size() * sizeof(float));
+        km->base()->output_sink = h_out_centroids;
+        if (km->hier) km->hier->TrainDevice(d_data, n, d_queries, n_queries);
+        else km->flat->TrainDevice(d_data, n, d_queries, n_queries);
         km->n_trained = n;
     });
 }
