@@ -72,6 +72,41 @@ def test_assign_full_clustered_data_exact_agreement(capi, ctx, oracle, blobs):
     assert gd.min() >= 0.0
 
 
+@pytest.mark.parametrize("n,k,d", [(70001, 1031, 96), (66000, 1100, 70), (70000, 1024, 33)])
+def test_assign_full_workgroup_tile_shape_never_changes_a_bit(capi, ctx, oracle, n, k, d):
+    """At least 1,024 tiles of 256 x 256 select the large workgroup shape, fewer the 128 x 128 one.  Both accumulate
+    every dot product in the same order, so one call over all points and calls over slices of 8,192 points must
+    return identical bits (ragged n and k, rows that are not 16-byte aligned, a trailing partial slice of d)."""
+    g = np.random.default_rng(n + k + d)
+    X = g.standard_normal((n, d)).astype(np.float32)
+    C = g.standard_normal((k, d)).astype(np.float32)
+    gi, gd, _ = _assign_full(capi, ctx, X, C)
+    for i0 in range(0, n, 8192):
+        si, sd, _ = _assign_full(capi, ctx, X[i0:i0 + 8192], C)
+        assert np.array_equal(gi[i0:i0 + 8192], si) and np.array_equal(gd[i0:i0 + 8192], sd)
+    m = 4000  # and the oracle on the last points (the ragged last tile)
+    bi, bbest, bsecond = oracle.brute_force(X[-m:], C)
+    tie = (bsecond - bbest) <= 1e-4 * np.maximum(bbest, 1e-12)
+    assert np.all((gi[-m:] == bi) | tie)
+    assert np.allclose(gd[-m:], bbest, rtol=1e-4, atol=1e-5)
+
+
+def test_rotate_large_tile_shape_equals_small_tile_shape(capi, ctx, oracle):
+    n, d = 270000, 256  # 1,055 tiles of 256 x 256
+    Q = oracle.rotation_matrix(d, seed=7)
+    X = np.random.default_rng(4).standard_normal((n, d)).astype(np.float32)
+    dX, dQ, dR = ctx.array(X), ctx.array(Q), ctx.empty((n, d))
+    capi.check(ctx.lib.skm_rotate(ctx.handle, dX.ptr, n, d, dQ.ptr, dR.ptr))
+    R = dR.download()
+    m = 5000
+    dS = ctx.empty((m, d))
+    capi.check(ctx.lib.skm_rotate(ctx.handle, dX.ptr + (n - m) * d * 4, m, d, dQ.ptr, dS.ptr))
+    assert np.array_equal(R[-m:], dS.download())
+    assert np.abs(R[:m] - X[:m].astype(np.float64) @ Q.astype(np.float64).T).max() < 1e-5
+    for a in (dX, dQ, dR, dS):
+        a.free()
+
+
 def test_assign_full_duplicate_centroids_take_lowest_index(capi, ctx):
     """Exact ties resolve to the lowest index inside a batch (minCoeff) and across batches (strict <)."""
     g = np.random.default_rng(3)
