@@ -50,7 +50,7 @@ static int fill_operands(GemmOperands& g, const float* A, int M, int64_t lda, co
 template <bool VEC, bool DIST, class S>
 __global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_store_kernel(
     GemmOperands g, float* __restrict__ out, int64_t ldo, const float* __restrict__ rn,
-    const float* __restrict__ cn
+    const float* __restrict__ cn, int wide_out
 ) {
     extern __shared__ float lds[];
     int tm, tn;
@@ -58,10 +58,68 @@ __global__ __launch_bounds__(S::THREADS, S::WG_PER_CU) void gemm_store_kernel(
     WaveAccT<S::FM, S::FN> acc;
     gemm_tile<VEC, S>(g, tm, tn, lds, acc);
 
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int m0 = tm * S::TM + (wave / S::WN) * S::WAVE_M;
-    const int n0 = tn * S::TN + (wave % S::WN) * S::WAVE_N;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / S::WN, wn = wave % S::WN;
+    const int m0 = tm * S::TM + wm * S::WAVE_M;
+    const int n0 = tn * S::TN + wn * S::WAVE_N;
+    if (wide_out) {
+        // Output rows are 16-byte aligned: the tile goes out through LDS, one block of 32 rows per wavefront row
+        // at a time, so that every store instruction writes whole 16-byte pieces of contiguous row segments
+        // (1 KiB per wavefront with the large shape) instead of 128-byte fragments of two rows.  Past the last
+        // barrier of the tile loop no wavefront reads the operand stages any more.
+        constexpr int PASS_ROWS = S::WM * 32;
+        constexpr int LDW = S::TN + 8;  // rows 4 apart land 32 banks apart: the 64 lanes of a store hit 64 banks
+        constexpr int LANES_PER_ROW = S::TN / 4;
+        constexpr int ROWS_PER_ITER = S::THREADS / LANES_PER_ROW;
+        static_assert(PASS_ROWS * LDW <= S::LDS_FLOATS, "staging block must fit the operand stages");
+        float cnv[S::FN];
+#pragma unroll
+        for (int nb = 0; nb < S::FN; ++nb) {
+            const int n = n0 + acc_col(nb, lane);
+            cnv[nb] = (DIST && n < g.N) ? cn[n] : 0.0f;
+        }
+#pragma unroll
+        for (int mb = 0; mb < S::FM; ++mb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = acc_row(0, r, lane);  // within the 32-row block
+                float rnv = 0.0f;
+                if (DIST) {
+                    const int m = m0 + mb * 32 + row;
+                    rnv = rn[m < g.M ? m : g.M - 1];
+                }
+#pragma unroll
+                for (int nb = 0; nb < S::FN; ++nb) {
+                    float v = acc.v[mb][nb][r];
+                    if (DIST) v = fmaf(-2.0f, v, rnv) + cnv[nb];
+                    lds[(wm * 32 + row) * LDW + wn * S::WAVE_N + acc_col(nb, lane)] = v;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < PASS_ROWS / ROWS_PER_ITER; ++it) {
+                const int rl = it * ROWS_PER_ITER + tid / LANES_PER_ROW;
+                const int c4 = (tid % LANES_PER_ROW) * 4;
+                const int m = tm * S::TM + (rl / 32) * S::WAVE_M + mb * 32 + (rl % 32);
+                const int n = tn * S::TN + c4;
+                if (m < g.M && n < g.N) {
+                    const floatx4 v4 = *reinterpret_cast<const floatx4*>(&lds[rl * LDW + c4]);
+                    float* dst = out + (int64_t) m * ldo + n;
+                    if (n + 3 < g.N) {
+                        *reinterpret_cast<floatx4*>(dst) = v4;
+                    } else {
+                        dst[0] = v4.x;
+                        if (n + 1 < g.N) dst[1] = v4.y;
+                        if (n + 2 < g.N) dst[2] = v4.z;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        return;
+    }
 #pragma unroll
     for (int nb = 0; nb < S::FN; ++nb) {
         const int n = n0 + acc_col(nb, lane);
@@ -93,14 +151,15 @@ static int launch_gemm_store_shape(skm_ctx* ctx, const float* A, int M, int64_t 
     const bool dist = row_norm != nullptr && col_norm != nullptr;
     const size_t lds_bytes = S::LDS_FLOATS * sizeof(float);
     dim3 grid((unsigned) (g.tiles_m * g.tiles_n)), block(S::THREADS);
+    const int wide_out = (reinterpret_cast<uintptr_t>(out) % 16 == 0 && ldo % 4 == 0) ? 1 : 0;
     if (vec && dist)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<true, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+        SKM_LAUNCH_GEMM((gemm_store_kernel<true, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm, wide_out);
     else if (vec)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<true, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+        SKM_LAUNCH_GEMM((gemm_store_kernel<true, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm, wide_out);
     else if (dist)
-        SKM_LAUNCH_GEMM((gemm_store_kernel<false, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+        SKM_LAUNCH_GEMM((gemm_store_kernel<false, true, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm, wide_out);
     else
-        SKM_LAUNCH_GEMM((gemm_store_kernel<false, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm);
+        SKM_LAUNCH_GEMM((gemm_store_kernel<false, false, S>), grid, block, lds_bytes, ctx->stream, g, out, ldo, row_norm, col_norm, wide_out);
     return check_hip(hipGetLastError(), "gemm_store_kernel launch");
 }
 
