@@ -25,11 +25,16 @@ static int allow_large_lds(Kernel kernel, size_t bytes) {
     } while (0)
 
 // The large shape pays off once its tiles fill the chip a few times over; below that (hierarchical fine
-// clusterings, tests) the small shape wastes less on partial tiles and keeps more workgroups in flight.
+// clusterings, tests) the small shape keeps more workgroups in flight.  Its loop is about 4.5 % faster per
+// flop, so it is also passed over when padding M and N to multiples of 256 instead of 128 adds more work
+// than that (k = 300 would be computed as 512 rows instead of 384).
 static bool use_big_tiles(int M, int N) {
     if (M < 192 || N < 192) return false;
+    auto padded = [](int v, int t) { return (double) ((v + t - 1) / t) * t; };
     const long long tiles = (long long) ((M + GemmBig::TM - 1) / GemmBig::TM) * ((N + GemmBig::TN - 1) / GemmBig::TN);
-    return tiles >= 1024;
+    const double work_big = padded(M, GemmBig::TM) * padded(N, GemmBig::TN);
+    const double work_small = padded(M, GemmSmall::TM) * padded(N, GemmSmall::TN);
+    return tiles >= 1024 && work_big <= 1.045 * work_small;
 }
 
 template <class S>

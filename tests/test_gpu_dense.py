@@ -72,7 +72,7 @@ def test_assign_full_clustered_data_exact_agreement(capi, ctx, oracle, blobs):
     assert gd.min() >= 0.0
 
 
-@pytest.mark.parametrize("n,k,d", [(70001, 1031, 96), (66000, 1100, 70), (70000, 1024, 33)])
+@pytest.mark.parametrize("n,k,d", [(70001, 1250, 96), (66000, 1500, 70), (70000, 1024, 33)])
 def test_assign_full_workgroup_tile_shape_never_changes_a_bit(capi, ctx, oracle, n, k, d):
     """At least 1,024 tiles of 256 x 256 select the large workgroup shape, fewer the 128 x 128 one.  Both accumulate
     every dot product in the same order, so one call over all points and calls over slices of 8,192 points must
