@@ -194,6 +194,9 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             dims_seen += SKM_H_DIM_SIZE;
             thr = best * a.ratios[dims_seen];
             cnt = compact_survivors(pos, acc, cnt, thr, lane);
+            // Only the incumbent is left: the best candidate stays what it is whatever the remaining steps do
+            // (pdxearch.h:140-143 applied after a step); with per-step accounting it keeps walking.
+            if (cnt == 1 && acct == nullptr && (uint32_t) (base + pos[0]) == prev_top_1) cnt = 0;
         }
 
         // ---- remaining vertical dimensions [d', V) from the dense auxiliary copy (pdxearch.h:183-216) ----
@@ -205,10 +208,21 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
                 const bool in = s < cnt;
                 const int cpos = in ? pos[s] : pos[0];
                 const float* cb = a.aux + (int64_t) (base + cpos) * V + dp;
+                // Four independent loads per operand in flight; the sum keeps the order t = sub, sub + 16, ...
                 float part = 0.0f;
-                for (int t = sub; t < left; t += 16) {
-                    const float e = xq[dp + t] - cb[t];
-                    part += e * e;
+                for (int t = sub; t < left; t += 64) {
+                    float xe[4], ce[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int tt = t + 16 * u;
+                        xe[u] = tt < left ? xq[dp + tt] : 0.0f;
+                        ce[u] = tt < left ? cb[tt] : 0.0f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float e = xe[u] - ce[u];
+                        part += e * e;
+                    }
                 }
                 part = group16_sum(part);
                 if (in && sub == 0) acc[s] += part;
@@ -318,10 +332,12 @@ template <bool VEC>
 __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListArgs a) {
     __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
     __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
+    __shared__ float s_parts[PRUNE_WAVES][16 * 8];  // [block of the group][survivor]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int p = blockIdx.x * PRUNE_WAVES + wave;
     if (p >= a.n) return;
+    float* parts = s_parts[wave];
     const uint32_t n_cand = a.cand_count[p];
     if (n_cand > a.cap) return;  // handled densely by the caller
     uint16_t* pos = s_pos[wave];
@@ -377,43 +393,106 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
 
         const float* chunk = a.pdx + (int64_t) base * d;
         int dims_seen = dp;
-        float4 xv_next = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (n_hblocks > 0) xv_next = load_x4<VEC>(xq + V + sub * 4);
-        for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
-            if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
+        for (int hb = 0; hb < n_hblocks && cnt > 0;) {
             const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
-            // This block's slice of the point was requested one block ago; the next one is requested now.
-            const float4 xv = xv_next;
-            if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
-            // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
-            for (int s0 = 0; s0 < cnt; s0 += 16) {
-                float4 cv[4];
+            if (cnt <= 8) {
+                // Few survivors: a block per round trip would leave the wavefront waiting on one dependent gather
+                // after the other.  The 16 gather slots of a pass take G consecutive blocks of every survivor
+                // instead (G = 16 / cnt rounded to a power of two); the blocks are then applied in order by the
+                // lane that owns the survivor: add, test against the threshold of that depth, stop when pruned.
+                // Same additions in the same order as block by block; gathers past a survivor's end are wasted.
+                const int cp = cnt <= 1 ? 1 : (cnt <= 2 ? 2 : (cnt <= 4 ? 4 : 8));
+                const int shift = cnt <= 1 ? 0 : (cnt <= 2 ? 1 : (cnt <= 4 ? 2 : 3));
+                int G = 16 / cp;
+                if (G > n_hblocks - hb) G = n_hblocks - hb;
+                float4 cv[4], xs[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int s = s0 + 4 * u + grp;
-                    const int cpos = s < cnt ? pos[s] : pos[0];
-                    const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                    const int slot = 4 * u + grp;
+                    const int sv = slot & (cp - 1), g = slot >> shift;
+                    const bool valid = sv < cnt && g < G;
+                    const int cpos = valid ? pos[sv] : pos[0];
+                    const int gg = valid ? g : 0;
+                    const float* cb = blk + (int64_t) gg * m * SKM_H_DIM_SIZE + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
                     if (VEC) {
                         cv[u] = *reinterpret_cast<const float4*>(cb);
                     } else {
                         cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
                     }
+                    xs[u] = load_x4<VEC>(xq + V + (hb + gg) * SKM_H_DIM_SIZE + sub * 4);
                 }
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int s = s0 + 4 * u + grp;
+                    const int slot = 4 * u + grp;
+                    const int sv = slot & (cp - 1), g = slot >> shift;
                     float e, part = 0.0f;
-                    e = xv.x - cv[u].x; part += e * e;
-                    e = xv.y - cv[u].y; part += e * e;
-                    e = xv.z - cv[u].z; part += e * e;
-                    e = xv.w - cv[u].w; part += e * e;
+                    e = xs[u].x - cv[u].x; part += e * e;
+                    e = xs[u].y - cv[u].y; part += e * e;
+                    e = xs[u].z - cv[u].z; part += e * e;
+                    e = xs[u].w - cv[u].w; part += e * e;
                     part = group16_sum(part);
-                    if (s < cnt && sub == 0) acc[s] += part;
+                    if (sv < cnt && g < G && sub == 0) parts[g * 8 + sv] = part;
                 }
+                const bool owner = lane < cnt;
+                const uint16_t my_pos = owner ? pos[lane] : (uint16_t) 0;
+                float my_acc = owner ? acc[lane] : 0.0f;
+                bool alive = owner;
+                int done = 0;
+                for (; done < G; ++done) {
+                    const int entering = __popcll(__ballot(alive));
+                    if (entering == 0) break;
+                    if (acct && lane == 0) atomicAdd(&acct[1 + hb + done], (unsigned long long) entering);
+                    if (alive) my_acc += parts[done * 8 + lane];
+                    alive = alive && my_acc < best * a.ratios[dims_seen + (done + 1) * SKM_H_DIM_SIZE];
+                }
+                const unsigned long long mask = __ballot(alive);
+                if (alive) {
+                    const int slot = __popcll(mask & ((1ull << lane) - 1ull));
+                    pos[slot] = my_pos;
+                    acc[slot] = my_acc;
+                }
+                cnt = __popcll(mask);
+                hb += G;
+                dims_seen += G * SKM_H_DIM_SIZE;
+            } else {
+                if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
+                const float4 xv = load_x4<VEC>(xq + V + hb * SKM_H_DIM_SIZE + sub * 4);
+                // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
+                for (int s0 = 0; s0 < cnt; s0 += 16) {
+                    float4 cv[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int s = s0 + 4 * u + grp;
+                        const int cpos = s < cnt ? pos[s] : pos[0];
+                        const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                        if (VEC) {
+                            cv[u] = *reinterpret_cast<const float4*>(cb);
+                        } else {
+                            cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int s = s0 + 4 * u + grp;
+                        float e, part = 0.0f;
+                        e = xv.x - cv[u].x; part += e * e;
+                        e = xv.y - cv[u].y; part += e * e;
+                        e = xv.z - cv[u].z; part += e * e;
+                        e = xv.w - cv[u].w; part += e * e;
+                        part = group16_sum(part);
+                        if (s < cnt && sub == 0) acc[s] += part;
+                    }
+                }
+                hb += 1;
+                dims_seen += SKM_H_DIM_SIZE;
+                cnt = compact_survivors(pos, acc, cnt, best * a.ratios[dims_seen], lane);
             }
-            dims_seen += SKM_H_DIM_SIZE;
             thr = best * a.ratios[dims_seen];
-            cnt = compact_survivors(pos, acc, cnt, thr, lane);
+            // Only the incumbent is left: whatever the remaining steps do to it, the best candidate stays what
+            // it is (the rule of pdxearch.h:140-143, applied after a step as well as before the first one).  It
+            // would otherwise walk all remaining blocks alone, one dependent gather after the other.  With
+            // per-step accounting requested it keeps walking, so that the counts are those of the reference.
+            if (cnt == 1 && acct == nullptr && (uint32_t) (base + pos[0]) == prev_top_1) cnt = 0;
         }
         if (cnt > 0 && dp < V) {
             if (acct && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
@@ -423,10 +502,21 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
                 const bool in = s < cnt;
                 const int cpos = in ? pos[s] : pos[0];
                 const float* cb = a.aux + (int64_t) (base + cpos) * V + dp;
+                // Four independent loads per operand in flight; the sum keeps the order t = sub, sub + 16, ...
                 float part = 0.0f;
-                for (int t = sub; t < left; t += 16) {
-                    const float e = xq[dp + t] - cb[t];
-                    part += e * e;
+                for (int t = sub; t < left; t += 64) {
+                    float xe[4], ce[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int tt = t + 16 * u;
+                        xe[u] = tt < left ? xq[dp + tt] : 0.0f;
+                        ce[u] = tt < left ? cb[tt] : 0.0f;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float e = xe[u] - ce[u];
+                        part += e * e;
+                    }
                 }
                 part = group16_sum(part);
                 if (in && sub == 0) acc[s] += part;
