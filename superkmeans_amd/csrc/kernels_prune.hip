@@ -38,11 +38,18 @@ struct PruneArgs {
     int n, k, d, vertical_d, partial_d;
 };
 
+// Sum over each group of 16 consecutive lanes, returned in all of them.  Rotations inside a row of 16 lanes are
+// data-parallel primitives of the vector unit (no trip through the LDS crossbar); the pairing is that of a
+// butterfly over lane distances 8, 4, 2, 1, so every lane adds the same pairs in the same order.
+template <int N>
+__device__ __forceinline__ float row_ror(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float group16_sum(float v) {
-    v += __shfl_xor(v, 8);
-    v += __shfl_xor(v, 4);
-    v += __shfl_xor(v, 2);
-    v += __shfl_xor(v, 1);
+    v += row_ror<8>(v);
+    v += row_ror<4>(v);
+    v += row_ror<2>(v);
+    v += row_ror<1>(v);
     return v;
 }
 
