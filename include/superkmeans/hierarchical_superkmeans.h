@@ -253,7 +253,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         return this->GetOutputCentroids(hierarchical_config.unrotate_centroids);
     }
 
-    static constexpr size_t FINE_HELPERS_DEFAULT = 4;  // concurrent fine-phase problems when n_threads is 0
+    static constexpr size_t FINE_HELPERS_DEFAULT = 8;  // concurrent fine-phase problems when n_threads is 0
     static constexpr size_t FINE_HELPERS_MAX = 16;
 
     // What every fine-phase problem reads (device pointers of the owner, host tables) and where it writes.

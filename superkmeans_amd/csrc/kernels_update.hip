@@ -146,28 +146,34 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     }
 }
 
-// One workgroup per centroid; thread t owns columns 4t..4t+3 (+ blockDim * 4 ...).  Rows of the
-// segment are visited in ascending point id; `UNROLL` independent row loads are kept in flight.
-template <bool VEC>
+// `groups` workgroups per centroid, each owning a contiguous range of columns (thread t of a group owns
+// columns 4t..4t+3 of that range).  Rows of the segment are visited in ascending point id, so the sum of every
+// column is accumulated in the reference's order whatever the number of groups; `UNROLL` independent row
+// loads are kept in flight per thread.  With many centroids one group per centroid fills the chip; with few,
+// long segments (mesoclustering: 256 centroids over 10 M points) the columns are spread over several
+// workgroups and more rows are kept in flight.
+template <bool VEC, int UNROLL>
 __global__ __launch_bounds__(256) void segment_sum_kernel(
     const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
-    const uint32_t* __restrict__ offsets, float* __restrict__ sums
+    const uint32_t* __restrict__ offsets, float* __restrict__ sums, uint32_t groups
 ) {
-    const uint32_t c = blockIdx.x;
+    const uint32_t c = blockIdx.x / groups, g = blockIdx.x % groups;
     const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
     float* out = sums + (size_t) c * d;
     if (VEC) {
         const size_t d4 = d / 4;
-        for (size_t t = threadIdx.x; t < d4; t += blockDim.x) {
+        const size_t per = (d4 + groups - 1) / groups;
+        const size_t t_end = (g + 1) * per < d4 ? (g + 1) * per : d4;
+        for (size_t t = g * per + threadIdx.x; t < t_end; t += blockDim.x) {
             float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
             uint32_t j = j0;
-            for (; j + 16 <= j1; j += 16) {
-                float4 v[16];
+            for (; j + UNROLL <= j1; j += UNROLL) {
+                float4 v[UNROLL];
 #pragma unroll
-                for (int u = 0; u < 16; ++u)
+                for (int u = 0; u < UNROLL; ++u)
                     v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
 #pragma unroll
-                for (int u = 0; u < 16; ++u) {
+                for (int u = 0; u < UNROLL; ++u) {
                     acc.x += v[u].x;
                     acc.y += v[u].y;
                     acc.z += v[u].z;
@@ -197,7 +203,9 @@ __global__ __launch_bounds__(256) void segment_sum_kernel(
             reinterpret_cast<float4*>(out)[t] = acc;
         }
     } else {
-        for (size_t t = threadIdx.x; t < d; t += blockDim.x) {
+        const size_t per = (d + groups - 1) / groups;
+        const size_t t_end = (g + 1) * per < d ? (g + 1) * per : d;
+        for (size_t t = g * per + threadIdx.x; t < t_end; t += blockDim.x) {
             float acc = 0.0f;
             for (uint32_t j = j0; j < j1; ++j) acc += x[(size_t) sorted_ids[j] * d + t];
             out[t] = acc;
@@ -393,11 +401,20 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
     const size_t lanes = vec ? d / 4 : d;
-    unsigned threads = (unsigned) std::min<size_t>(256, ((lanes + 63) / 64) * 64);
-    if (vec)
-        hipLaunchKernelGGL(segment_sum_kernel<true>, dim3((unsigned) k), dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+    // Few centroids: spread the columns of a centroid over several workgroups of at least one wavefront until
+    // about 2,048 workgroups are in flight, and keep more rows in flight when segments are long on average.
+    size_t groups = 1;
+    while (k * groups < 2048 && lanes / (groups * 2) >= 64) groups *= 2;
+    const size_t per = (lanes + groups - 1) / groups;
+    unsigned threads = (unsigned) std::min<size_t>(256, ((per + 63) / 64) * 64);
+    dim3 grid((unsigned) (k * groups));
+    const bool long_segments = n / k >= 1024;
+    if (vec && long_segments)
+        hipLaunchKernelGGL((segment_sum_kernel<true, 32>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+    else if (vec)
+        hipLaunchKernelGGL((segment_sum_kernel<true, 16>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
     else
-        hipLaunchKernelGGL(segment_sum_kernel<false>, dim3((unsigned) k), dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+        hipLaunchKernelGGL((segment_sum_kernel<false, 16>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
     return check_hip(hipGetLastError(), "segment_sum_kernel launch");
 }
 
