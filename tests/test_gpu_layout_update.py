@@ -28,7 +28,10 @@ def test_pdxify_rejects_bad_split(capi, ctx):
 
 
 @pytest.mark.parametrize("n,d,k,nthreads", [(5000, 128, 100, 1), (20000, 256, 1000, 8), (3000, 50, 7, 3), (10000, 1024, 300, 8),
-                                            (70000, 64, 70000, 8), (257, 1536, 1, 2)])
+                                            (70000, 64, 70000, 8), (257, 1536, 1, 2),
+                                            # few centroids, long segments: columns of a centroid spread over several
+                                            # workgroups, 32 rows in flight per thread; the order of additions is the same
+                                            (40000, 1024, 9, 4), (50000, 512, 20, 2)])
 def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
     g = np.random.default_rng(n + d)
     X = g.standard_normal((n, d)).astype(np.float32)
