@@ -47,8 +47,28 @@ class UnitUniformDraws {
     explicit UnitUniformDraws(std::mt19937& rng) : rng_(rng), direct_(DirectFormMatches()) {}
     float operator()() {
         if (!direct_) return std::uniform_real_distribution<float>(0, 1)(rng_);
-        const float r = static_cast<float>(rng_()) * 0x1p-32f;
-        return r < 1.0f ? r : std::nextafter(1.0f, 0.0f);
+        return FromRaw(rng_());
+    }
+    // True when a draw is FromRaw(one 32-bit output of the engine); then `draw() < p` can be decided on the raw
+    // integer: FromRaw is monotone, so the accepted outputs are exactly those below AcceptBelow(p).
+    bool direct() const { return direct_; }
+    uint32_t raw() { return static_cast<uint32_t>(rng_()); }
+    static float FromRaw(const uint32_t r) {
+        const float u = static_cast<float>(r) * 0x1p-32f;
+        return u < 1.0f ? u : std::nextafter(1.0f, 0.0f);
+    }
+    // Number of 32-bit outputs r with FromRaw(r) < p (0 ... 2^32), found by bisection on the monotone predicate.
+    static uint64_t AcceptBelow(const float p) {
+        uint64_t lo = 0, hi = uint64_t(1) << 32;  // FromRaw(r) < p for r < lo, not for r >= hi
+        if (!(FromRaw(0) < p)) return 0;
+        if (FromRaw(0xffffffffu) < p) return hi;
+        lo = 1;
+        hi = 0xffffffffu;
+        while (lo < hi) {
+            const uint64_t mid = lo + (hi - lo) / 2;
+            if (FromRaw(static_cast<uint32_t>(mid)) < p) lo = mid + 1; else hi = mid;
+        }
+        return lo;
     }
 
   private:

@@ -505,23 +505,41 @@ class SuperKMeans {
         const auto accept_probability = [&](const size_t c) -> float {
             return (cluster_sizes[c] - 1.0) / (float) (n_samples_ - k);
         };
+        // With the direct form of the draws the test `draw < p` is decided on the engine's raw 32-bit output
+        // against an integer bound per cluster (same decisions, no float conversion in the walk).
         std::vector<float> prob;
+        std::vector<uint64_t> bound;
         UnitUniformDraws draw(rng);
+        const bool on_raw = draw.direct();
         for (size_t ci = 0; ci < k; ci++) {
             if (cluster_sizes[ci] != 0) continue;
             if (prob.empty()) {
                 prob.resize(k);
                 for (size_t c = 0; c < k; ++c) prob[c] = accept_probability(c);
+                if (on_raw) {
+                    bound.resize(k);
+                    for (size_t c = 0; c < k; ++c) bound[c] = UnitUniformDraws::AcceptBelow(prob[c]);
+                }
             }
             size_t cj;
-            for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
-                if (draw() < prob[cj]) break;
+            if (on_raw) {
+                for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
+                    if (draw.raw() < bound[cj]) break;
+                }
+            } else {
+                for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
+                    if (draw() < prob[cj]) break;
+                }
             }
             edits.push_back({0u, static_cast<uint32_t>(ci), static_cast<uint32_t>(cj), 0.0f});
             cluster_sizes[ci] = cluster_sizes[cj] / 2;
             cluster_sizes[cj] -= cluster_sizes[ci];
             prob[ci] = accept_probability(ci);
             prob[cj] = accept_probability(cj);
+            if (on_raw) {
+                bound[ci] = UnitUniformDraws::AcceptBelow(prob[ci]);
+                bound[cj] = UnitUniformDraws::AcceptBelow(prob[cj]);
+            }
             n_split++;
         }
         ApplyRowEdits(edits);
