@@ -43,6 +43,8 @@ static int fill_operands(GemmOperands& g, const float* A, int M, int64_t lda, co
     g.tiles_m = (M + S::TM - 1) / S::TM;
     g.tiles_n = (N + S::TN - 1) / S::TN;
     if ((long long) g.tiles_m * g.tiles_n > 0x7fffffffLL) return set_error(SKM_ERR_INVALID, "gemm grid too large");
+    // Operand rows are addressed with 32-bit byte offsets from the tile's first row (at most 256 rows).
+    if (lda > (int64_t(1) << 20) || ldb > (int64_t(1) << 20)) return set_error(SKM_ERR_INVALID, "gemm row stride above 2^20");
     return SKM_OK;
 }
 
