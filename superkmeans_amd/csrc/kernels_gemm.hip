@@ -309,8 +309,8 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
 //   group's fragments fetched ahead; workgroup barrier before the last group; first fragments of slice
 //   s + 1; last group; epilogue if the tile ends here.
 // FAST: rows are 16-byte aligned and hold at least round_up(d', 32) columns, so every slice is fetched
-// without guards; columns at or past d' in the last group are zeroed in the centroid fragments (finite
-// point values times zero add nothing).  Otherwise slices are fetched with guards (zeros past d').
+// without guards; columns at or past d' in the last group are zeroed in the fragments of both operands.
+// Otherwise slices are fetched with guards (zeros past d').
 // Workgroups of one XCD sweep the centroid tiles roughly in step and share them through that XCD's L2.
 template <bool FAST>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
@@ -502,12 +502,15 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
                 a0 = na0; a1 = na1; b0 = nb0; b1 = nb1;
             }
             if (FAST) {
-                // zero the centroid columns at or past d' in the last group of the tile's last slice
+                // zero the columns at or past d' in the last group of the tile's last slice (both operands, so that
+                // whatever lies there, even a non-finite value, contributes an exact zero)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const bool live = !last || last_col0 + i < g.K;
                     a0[i] = live ? a0[i] : 0.0f;
                     a1[i] = live ? a1[i] : 0.0f;
+                    b0[i] = live ? b0[i] : 0.0f;
+                    b1[i] = live ? b1[i] : 0.0f;
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
