@@ -172,11 +172,11 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             // This block's slice of the point was requested one block ago; the next one is requested now.
             const float4 xv = xv_next;
             if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
-            // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
-            for (int s0 = 0; s0 < cnt; s0 += 16) {
-                float4 cv[4];
+            // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.
+            for (int s0 = 0; s0 < cnt; s0 += 32) {
+                float4 cv[8];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < 8; ++u) {
                     const int s = s0 + 4 * u + grp;
                     const int cpos = s < cnt ? pos[s] : pos[0];
                     const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
                     }
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+                for (int u = 0; u < 8; ++u) {
                     const int s = s0 + 4 * u + grp;
                     float e, part = 0.0f;
                     e = xv.x - cv[u].x; part += e * e;
