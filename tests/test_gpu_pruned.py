@@ -46,7 +46,12 @@ def _setup(oracle, blobs, n, d, k, seed, std=0.3):
 
 
 @pytest.mark.parametrize("n,d,k,partial_d", [(4000, 128, 300, 32), (6000, 256, 1500, 32), (3000, 768, 1100, 96),
-                                             (4000, 1024, 2500, 128), (1500, 600, 1030, 77), (1000, 132, 260, 23)])
+                                             (4000, 1024, 2500, 128), (1500, 600, 1030, 77), (1000, 132, 260, 23),
+                                             # shapes of the slice pipeline of the candidate kernel: one centroid tile
+                                             # of two slices; two tiles of one masked slice; a last slice of a single
+                                             # masked group; round_up(d', 32) equal to the row length; unaligned rows
+                                             (600, 128, 100, 64), (300, 256, 129, 17), (700, 192, 300, 33),
+                                             (500, 128, 257, 63), (400, 130, 200, 40)])
 def test_pruned_matches_oracle(capi, ctx, oracle, blobs, n, d, k, partial_d):
     X, C, prev = _setup(oracle, blobs, n, d, k, seed=n + d)
     ratios = oracle.ratios(d, 1.5)
