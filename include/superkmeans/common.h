@@ -3,6 +3,7 @@
 // algorithm (batch shapes decide tie-breaking and threshold schedules), not tuning knobs.
 #pragma once
 
+#include <algorithm>
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
@@ -94,6 +95,79 @@ class UnitUniformDraws {
     }
     std::mt19937& rng_;
     const bool direct_;
+};
+
+// The output stream of std::mt19937 (the 32-bit Mersenne Twister of Matsumoto and Nishimura with the standard's
+// seeding recurrence), produced 624 outputs at a time into an array.  The cluster-splitting walk tests millions
+// of consecutive draws against a table; on an array that test is a vector compare instead of one engine call
+// per draw.  Outputs, in order, are exactly those of std::mt19937(seed).
+class Mt19937Blocks {
+  public:
+    static constexpr size_t BLOCK = 624;
+    explicit Mt19937Blocks(const uint32_t seed) {
+        state_[0] = seed;
+        for (uint32_t i = 1; i < BLOCK; ++i) state_[i] = 1812433253u * (state_[i - 1] ^ (state_[i - 1] >> 30)) + i;
+    }
+    // Unconsumed outputs of the current block (refilled when none is left) and their count.
+    const uint32_t* Peek() {
+        if (pos_ == BLOCK) Refill();
+        return out_ + pos_;
+    }
+    size_t Remaining() const { return BLOCK - pos_; }
+    void Consume(const size_t count) { pos_ += count; }
+
+    /**
+     * The walk of SplitClusters for one empty cluster: starting at cluster 0 and cycling over [0, k), one draw
+     * per visited cluster, returns the first cluster whose draw is below its bound.  bound[c] is the number of
+     * 32-bit outputs accepted for cluster c and must be below 2^32 for every c and positive for at least one.
+     */
+    size_t WalkToFirstAccepted(const uint32_t* bound, const size_t k) {
+        size_t c = 0;
+        for (;;) {
+            const uint32_t* r = Peek();
+            const size_t len = std::min(Remaining(), k - c);
+            const uint32_t* b = bound + c;
+            size_t i = 0;
+            for (; i + 16 <= len; i += 16) {
+                uint32_t any = 0;
+                for (size_t j = 0; j < 16; ++j) any |= static_cast<uint32_t>(r[i + j] < b[i + j]);
+                if (any) break;
+            }
+            for (; i < len; ++i) {
+                if (r[i] < b[i]) {
+                    Consume(i + 1);
+                    return c + i;
+                }
+            }
+            Consume(len);
+            c += len;
+            if (c == k) c = 0;
+        }
+    }
+
+  private:
+    static uint32_t Twist(const uint32_t upper, const uint32_t lower, const uint32_t far) {
+        const uint32_t y = (upper & 0x80000000u) | (lower & 0x7fffffffu);
+        return far ^ (y >> 1) ^ ((lower & 1u) ? 0x9908b0dfu : 0u);
+    }
+    void Refill() {
+        constexpr size_t M = 397;
+        for (size_t i = 0; i < BLOCK - M; ++i) state_[i] = Twist(state_[i], state_[i + 1], state_[i + M]);
+        for (size_t i = BLOCK - M; i < BLOCK - 1; ++i) state_[i] = Twist(state_[i], state_[i + 1], state_[i + M - BLOCK]);
+        state_[BLOCK - 1] = Twist(state_[BLOCK - 1], state_[0], state_[M - 1]);
+        for (size_t i = 0; i < BLOCK; ++i) {
+            uint32_t y = state_[i];
+            y ^= y >> 11;
+            y ^= (y << 7) & 0x9d2c5680u;
+            y ^= (y << 15) & 0xefc60000u;
+            y ^= y >> 18;
+            out_[i] = y;
+        }
+        pos_ = 0;
+    }
+    uint32_t state_[BLOCK];
+    uint32_t out_[BLOCK];
+    size_t pos_ = BLOCK;
 };
 
 enum class DistanceFunction : uint8_t { l2, dp };

@@ -506,11 +506,19 @@ class SuperKMeans {
             return (cluster_sizes[c] - 1.0) / (float) (n_samples_ - k);
         };
         // With the direct form of the draws the test `draw < p` is decided on the engine's raw 32-bit output
-        // against an integer bound per cluster (same decisions, no float conversion in the walk).
+        // against an integer bound per cluster (same decisions, no float conversion in the walk), and the
+        // outputs come in blocks so that the walk scans arrays.  A bound of 2^32 (p >= 1, which sizes of a
+        // real clustering do not produce) does not fit the table: then every draw goes through the engine.
         std::vector<float> prob;
-        std::vector<uint64_t> bound;
+        std::vector<uint32_t> bound;
         UnitUniformDraws draw(rng);
-        const bool on_raw = draw.direct();
+        Mt19937Blocks blocks(static_cast<uint32_t>(config.seed));
+        bool on_raw = draw.direct();
+        const auto set_bound = [&](const size_t c) -> bool {
+            const uint64_t b = UnitUniformDraws::AcceptBelow(prob[c]);
+            bound[c] = static_cast<uint32_t>(b);
+            return b <= 0xffffffffu;
+        };
         for (size_t ci = 0; ci < k; ci++) {
             if (cluster_sizes[ci] != 0) continue;
             if (prob.empty()) {
@@ -518,14 +526,17 @@ class SuperKMeans {
                 for (size_t c = 0; c < k; ++c) prob[c] = accept_probability(c);
                 if (on_raw) {
                     bound.resize(k);
-                    for (size_t c = 0; c < k; ++c) bound[c] = UnitUniformDraws::AcceptBelow(prob[c]);
+                    bool any = false;
+                    for (size_t c = 0; c < k; ++c) {
+                        on_raw = set_bound(c) && on_raw;
+                        any = any || bound[c] != 0;
+                    }
+                    on_raw = on_raw && any;  // with no acceptable cluster the walk below never ends, as in the reference
                 }
             }
             size_t cj;
             if (on_raw) {
-                for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
-                    if (draw.raw() < bound[cj]) break;
-                }
+                cj = blocks.WalkToFirstAccepted(bound.data(), k);
             } else {
                 for (cj = 0; true; cj = (cj + 1 == k) ? 0 : cj + 1) {
                     if (draw() < prob[cj]) break;
@@ -537,8 +548,9 @@ class SuperKMeans {
             prob[ci] = accept_probability(ci);
             prob[cj] = accept_probability(cj);
             if (on_raw) {
-                bound[ci] = UnitUniformDraws::AcceptBelow(prob[ci]);
-                bound[cj] = UnitUniformDraws::AcceptBelow(prob[cj]);
+                // probabilities only shrink (a split halves the donor), so the bounds keep fitting
+                set_bound(ci);
+                set_bound(cj);
             }
             n_split++;
         }
