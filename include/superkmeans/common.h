@@ -263,6 +263,10 @@ class Buffer {
     void Upload(const T* host, size_t count, size_t dst_offset = 0) {
         Check(skm_upload(ctx_, ptr_ + dst_offset, host, count * sizeof(T)));
     }
+    // Copy on the transfer stream: queued work keeps running, later work waits (skm_upload_overlapped).
+    void UploadOverlapped(const T* host, size_t count, size_t dst_offset = 0) {
+        Check(skm_upload_overlapped(ctx_, ptr_ + dst_offset, host, count * sizeof(T)));
+    }
     void Download(T* host, size_t count, size_t src_offset = 0) const {
         Check(skm_download(ctx_, host, ptr_ + src_offset, count * sizeof(T)));
     }

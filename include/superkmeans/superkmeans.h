@@ -16,6 +16,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <functional>
 #include <iostream>
 #include <memory>
 #include <numeric>
@@ -165,17 +166,34 @@ class SuperKMeans {
         return TrainImpl(d_data, n, d_queries, n_queries, /*on_device=*/true);
     }
 
-    /** Exact nearest-centroid assignment; vectors and centroids must be in the same space. */
+    /**
+     * Exact nearest-centroid assignment; vectors and centroids must be in the same space.  The vectors go to the
+     * device in slabs of rows and every slab is searched while the next one is on its way.
+     */
     [[nodiscard]] std::vector<uint32_t> Assign(const vector_value_t* vectors, const vector_value_t* centroids,
                                                const size_t n_vectors, const size_t n_centroids) {
         dbuf<float> d_v(ctx, n_vectors * d), d_c(ctx, n_centroids * d);
-        d_v.Upload(vectors, n_vectors * d);
         d_c.Upload(centroids, n_centroids * d);
         dbuf<uint32_t> d_out(ctx, n_vectors);
-        AssignDevice(d_v.get(), d_c.get(), n_vectors, n_centroids, d_out.get());
+        dbuf<float> v_norms(ctx, n_vectors), c_norms(ctx, n_centroids), dist(ctx, n_vectors);
+        hip::Check(skm_norms(ctx, d_c.get(), n_centroids, d, d, c_norms.get()));
+        const size_t slab = UploadSlabRows();
+        for (size_t r0 = 0; r0 < n_vectors; r0 += slab) {
+            const size_t m = std::min(slab, n_vectors - r0);
+            d_v.UploadOverlapped(vectors + r0 * d, m * d, r0 * d);
+            hip::Check(skm_norms(ctx, d_v.get() + r0 * d, m, d, d, v_norms.get() + r0));
+            hip::Check(skm_assign_full(ctx, d_v.get() + r0 * d, m, d_c.get(), n_centroids, d, v_norms.get() + r0,
+                                       c_norms.get(), d_out.get() + r0, dist.get() + r0));
+        }
         std::vector<uint32_t> result(n_vectors);
         d_out.Download(result.data(), n_vectors);
         return result;
+    }
+
+    // Rows per slab of a host-to-device transfer that overlaps with compute: 256 MiB of rows, a multiple of 256.
+    size_t UploadSlabRows() const {
+        const size_t rows = (size_t(256) << 20) / (d * sizeof(float));
+        return std::max<size_t>(256, rows / 256 * 256);
     }
 
     /** Assign on device-resident inputs; writes n_vectors indices to d_out_assignments (asynchronous). */
@@ -355,13 +373,32 @@ class SuperKMeans {
         }
 
         const bool rotate = !config.data_already_rotated;
-        // The rotation of the training matrix is queued first so that it runs on the device while the host
-        // draws the initial centroids; the two steps share no state (each seeds its own mt19937).
-        const float* data_to_cluster = SampleAndRotateVectors(data, n, n_samples, rotate, on_device);
-        GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
-        // prev_centroids <- rotated initial centroids; horizontal_centroids still holds the raw rows.
-        RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
-        hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, d, data_norms.get()));
+        const float* data_to_cluster = nullptr;
+        first_search_done = false;
+        if (!on_device && n_samples == n && config.iters > 0) {
+            // Host rows that are all used: they reach the device in slabs, and every slab is rotated and searched
+            // against the initial centroids (the first iteration is always exact) while the next one is on its
+            // way.  The initial centroids come first for that; they are rows of the host matrix.
+            GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
+            RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
+            hip::Check(skm_norms(ctx, prev_centroids.get(), n_clusters, d, d, centroid_norms.get()));
+            data_to_cluster = SampleAndRotateVectors(
+                data, n, n_samples, rotate, on_device, [&](const float* d_rows, const size_t r0, const size_t m) {
+                    hip::Check(skm_norms(ctx, d_rows, m, d, d, data_norms.get() + r0));
+                    hip::Check(skm_assign_full(ctx, d_rows, m, prev_centroids.get(), n_clusters, d,
+                                               data_norms.get() + r0, centroid_norms.get(),
+                                               d_assignments.get() + r0, distances.get() + r0));
+                });
+            first_search_done = true;
+        } else {
+            // The rotation of the training matrix is queued first so that it runs on the device while the host
+            // draws the initial centroids; the two steps share no state (each seeds its own mt19937).
+            data_to_cluster = SampleAndRotateVectors(data, n, n_samples, rotate, on_device);
+            GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
+            // prev_centroids <- rotated initial centroids; horizontal_centroids still holds the raw rows.
+            RotateOrCopy(horizontal_centroids.get(), prev_centroids.get(), n_clusters, rotate);
+            hip::Check(skm_norms(ctx, data_to_cluster, n_samples, d, d, data_norms.get()));
+        }
         n_tracked_queries = 0;
         if (n_queries) PrepareQueries(data_to_cluster, queries, n_queries, on_device);
 
@@ -410,7 +447,9 @@ class SuperKMeans {
                       std::vector<SuperKMeansIterationStats>& target_stats) {
         if (!is_first_iter) horizontal_centroids.swap(prev_centroids);
         uint64_t not_pruned_total = 0;
-        if (gemm_only) {
+        if (gemm_only && is_first_iter && first_search_done) {
+            first_search_done = false;  // Train searched slab by slab while the rows were uploaded
+        } else if (gemm_only) {
             hip::Check(skm_norms(ctx, prev_centroids.get(), k, d, d, centroid_norms.get()));
             hip::Check(skm_assign_full(ctx, data_to_cluster, n_samples_, prev_centroids.get(), k, d, data_norms.get(),
                                        centroid_norms.get(), d_assignments.get(), distances.get()));
@@ -785,7 +824,8 @@ class SuperKMeans {
      * used in place.
      */
     const float* SampleAndRotateVectors(const vector_value_t* data, const size_t n, const size_t n_samples_,
-                                        const bool rotate, const bool on_device) {
+                                        const bool rotate, const bool on_device,
+                                        const std::function<void(const float*, size_t, size_t)>& after_slab = {}) {
         const bool sample = n_samples_ < n;
         if (sample) {
             std::mt19937 rng(config.seed);
@@ -794,6 +834,23 @@ class SuperKMeans {
             std::shuffle(sampled_indices.get(), sampled_indices.get() + n, rng);
         }
         if (on_device && !sample && !rotate) return data;
+        if (!on_device && !sample) {
+            // All host rows in order: slab after slab on the transfer stream, each one rotated (and handed to
+            // after_slab: training rows on the device, first row, count) while the next is copied.
+            training_data.Reset(ctx, n_samples_ * d);
+            dbuf<float> raw;
+            if (rotate) raw.Reset(ctx, n_samples_ * d);
+            dbuf<float>& landing = rotate ? raw : training_data;
+            const size_t slab = UploadSlabRows();
+            for (size_t r0 = 0; r0 < n_samples_; r0 += slab) {
+                const size_t m = std::min(slab, n_samples_ - r0);
+                landing.UploadOverlapped(data + r0 * d, m * d, r0 * d);
+                if (rotate) pruner->Rotate(raw.get() + r0 * d, training_data.get() + r0 * d, m);
+                if (after_slab) after_slab(training_data.get() + r0 * d, r0, m);
+            }
+            if (rotate) hip::Check(skm_sync(ctx));  // `raw` is released on return
+            return training_data.get();
+        }
         dbuf<float> staged;  // raw rows on the device, in training order
         const float* d_raw = nullptr;
         if (on_device && !sample) {
@@ -808,18 +865,14 @@ class SuperKMeans {
             d_raw = staged.get();
         } else {
             staged.Reset(ctx, n_samples_ * d);
-            if (!sample) {
-                staged.Upload(data, n_samples_ * d);
-            } else {
-                // Gather on the host in slabs so the staging buffer stays small.
-                const size_t slab = std::max<size_t>(1, (size_t(64) << 20) / (d * sizeof(float)));
-                std::vector<float> host(std::min(slab, n_samples_) * d);
-                for (size_t i0 = 0; i0 < n_samples_; i0 += slab) {
-                    const size_t m = std::min(slab, n_samples_ - i0);
-                    for (size_t i = 0; i < m; ++i)
-                        std::memcpy(&host[i * d], data + sampled_indices[i0 + i] * d, sizeof(float) * d);
-                    staged.Upload(host.data(), m * d, i0 * d);
-                }
+            // Gather on the host in slabs so the staging buffer stays small.
+            const size_t slab = std::max<size_t>(1, (size_t(64) << 20) / (d * sizeof(float)));
+            std::vector<float> host(std::min(slab, n_samples_) * d);
+            for (size_t i0 = 0; i0 < n_samples_; i0 += slab) {
+                const size_t m = std::min(slab, n_samples_ - i0);
+                for (size_t i = 0; i < m; ++i)
+                    std::memcpy(&host[i * d], data + sampled_indices[i0 + i] * d, sizeof(float) * d);
+                staged.Upload(host.data(), m * d, i0 * d);
             }
             d_raw = staged.get();
         }
@@ -849,6 +902,7 @@ class SuperKMeans {
     uint32_t partial_d = 0;
 
     bool trained = false;
+    bool first_search_done = false;  // Train's first exact search ran during the upload of the rows
     size_t n_split = 0;
     uint32_t vertical_d = 0;
     float prev_cost = 0.0f;

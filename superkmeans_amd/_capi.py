@@ -29,6 +29,7 @@ _PROTOTYPES = {
     "skm_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "skm_free": (c_int, [c_void_p, c_void_p]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "skm_upload_overlapped": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_download": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_fill_u32": (c_int, [c_void_p, c_void_p, c_uint32, c_size_t]),

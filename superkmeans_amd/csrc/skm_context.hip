@@ -168,6 +168,12 @@ int skm_ctx_destroy(skm_ctx* ctx) {
     for (int i = 0; i < 4; ++i)
         if (ctx->ws[i]) (void) hipFree(ctx->ws[i]);
     if (ctx->h_pinned) (void) hipHostFree(ctx->h_pinned);
+    if (ctx->copy_stream) {
+        (void) hipStreamSynchronize(ctx->copy_stream);
+        for (auto e : ctx->copy_done)
+            if (e) (void) hipEventDestroy(e);
+        (void) hipStreamDestroy(ctx->copy_stream);
+    }
     (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     return SKM_OK;
@@ -209,6 +215,34 @@ int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
     SKM_REQUIRE(d_dst && h_src, "null pointer");
     SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->stream));
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SKM_OK;
+}
+
+int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    if (bytes == 0) return SKM_OK;
+    SKM_REQUIRE(d_dst && h_src, "null pointer");
+    SKM_HIP_TRY(hipSetDevice(ctx->device));
+    if (!ctx->copy_stream) {
+        hipStream_t s = nullptr;
+        SKM_HIP_TRY(hipStreamCreate(&s));
+        for (auto& e : ctx->copy_done) {
+            const hipError_t rc = hipEventCreateWithFlags(&e, hipEventDisableTiming);
+            if (rc != hipSuccess) {
+                for (auto& made : ctx->copy_done) {
+                    if (made) (void) hipEventDestroy(made);
+                    made = nullptr;
+                }
+                (void) hipStreamDestroy(s);
+                return check_hip(rc, "hipEventCreateWithFlags");
+            }
+        }
+        ctx->copy_stream = s;
+    }
+    hipEvent_t done = ctx->copy_done[ctx->copy_seq++ % 8];
+    SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->copy_stream));
+    SKM_HIP_TRY(hipEventRecord(done, ctx->copy_stream));
+    SKM_HIP_TRY(hipStreamWaitEvent(ctx->stream, done, 0));
     return SKM_OK;
 }
 

@@ -23,6 +23,10 @@ struct skm_pending_interval {
 struct skm_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
+    // Transfer stream of skm_upload_overlapped (created on first use) and the events that order it before `stream`.
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t copy_done[8] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    unsigned copy_seq = 0;
     size_t workspace_limit = size_t(24) << 30;
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
     void* ws[4] = {nullptr, nullptr, nullptr, nullptr};

@@ -179,6 +179,36 @@ def test_train_device_resident_equals_host_path(capi, ctx, blobs):
     a.close(), b.close()
 
 
+def test_host_rows_arriving_in_slabs_give_the_device_resident_result(capi, ctx):
+    """Train and Assign on host pointers upload the rows in 256 MiB slabs and rotate / search every slab while the
+    next one is copied (the first, exact iteration of Train runs that way).  Three slabs with a ragged last one:
+    centroids, statistics, assignments and distances equal those of the device-resident path bit for bit."""
+    n, d, k = 80000, 2048, 300
+    km = capi.KMeans(k, d, iters=3, sampling_fraction=1.0, early_termination=0)
+    dX = km.ctx.empty((n, d))
+    capi.check(km.lib.skm_synth_gaussian_mixture(km.ctx.handle, dX.ptr, n, d, 0, k, 11, 12, 1.0, 0.3, 0.0, 0))
+    X = dX.download()
+    assert (256 << 20) // (d * 4) * 2 < n  # more than two slabs
+    Cd = km.train_device(dX, n)
+    kh = capi.KMeans(k, d, iters=3, sampling_fraction=1.0, early_termination=0)
+    Ch = kh.train(X)
+    assert np.array_equal(Cd, Ch)
+    sd, sh = km.stats(), kh.stats()
+    assert [(s.objective, s.shift, s.split, s.partial_d, s.not_pruned_pct) for s in sd] == \
+           [(s.objective, s.shift, s.split, s.partial_d, s.not_pruned_pct) for s in sh]
+    assert np.array_equal(km.assignments(n), kh.assignments(n))
+    dC, dOut = km.ctx.array(Cd), km.ctx.empty(n, np.uint32)
+    km.assign_device(dX, dC, n, k, dOut)
+    assert np.array_equal(dOut.download(), kh.assign(X, Ch))
+    # rows that are already rotated skip the rotation but take the same slab path
+    kr = capi.KMeans(k, d, iters=2, sampling_fraction=1.0, early_termination=0, data_already_rotated=1)
+    kq = capi.KMeans(k, d, iters=2, sampling_fraction=1.0, early_termination=0, data_already_rotated=1)
+    assert np.array_equal(kr.train(X), kq.train_device(dX, n))
+    for o in (dX, dC, dOut):
+        o.free()
+    km.close(), kh.close(), kr.close(), kq.close()
+
+
 def test_reproducible_and_exceptions(capi, ctx, blobs):
     n, d, k = 5000, 128, 260
     X = blobs(n, d, k, seed=2)
