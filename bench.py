@@ -8,7 +8,8 @@ L2-normalised, generated directly in HBM.
 One "step" is one Assign() pass (exact nearest centroid of every point) with points and centroids
 resident in HBM; `value` is points per second over the timed steps.  The same run also times one
 Train() (rotation + 1 GEMM-only iteration + pruned iterations, data resident in HBM) and reports
-seconds per iteration and the per-stage device times next to their rooflines.  The CPU baseline is
+seconds per iteration and the per-stage device times next to their rooflines, and repeats Assign and
+Train on host pointers (`host_pointers`: the transfer-inclusive times, never `value`).  The CPU baseline is
 the CPU oracle (OpenMP + BLAS restatement of the reference path) on a bounded prefix of the same
 points, on the host cores of the same box.
 
@@ -51,6 +52,8 @@ def main():
     ap.add_argument("--cpu-train-points", type=int, default=65536)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-train", action="store_true")
+    ap.add_argument("--no-host-pointers", action="store_true",
+                    help="skip the PCIe-inclusive leg (Assign and Train called with host pointers)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain row-copy kernel of known size (1 GiB read + 1 GiB write) three times; "
                          "used to scale the FETCH_SIZE / WRITE_SIZE hardware counters")
@@ -182,6 +185,27 @@ def main():
                 "traffic": MEASURED_TRAFFIC_BYTES.get((n, d, k)), "avg_launch_ms": round(gemm_avg_ms, 3), "flops_per_launch": flops_per_launch}
     gpu_assign = dOut.download()
 
+    # ---- PCIe-inclusive leg (reported beside `value`, never as it): the same calls on host pointers ----
+    host_pointers = None
+    if not args.no_host_pointers:
+        Xhost = dX.download()
+        km.assign(Xhost[: min(n, 4096)], centroids)  # buffers of the host path touched once
+        t0 = time.perf_counter()
+        host_assign = km.assign(Xhost, centroids)
+        host_assign_s = time.perf_counter() - t0
+        host_pointers = {"assign_ms": round(host_assign_s * 1e3, 1), "assign_points_per_s": round(n / host_assign_s, 1),
+                         "assign_equals_resident": bool(np.array_equal(host_assign, gpu_assign)),
+                         "note": "pageable host rows, uploaded in 256 MiB slabs on a transfer stream while the "
+                                 "previous slab is searched"}
+        if not args.no_train:
+            kmh = _capi.KMeans(k, d, **cfg)
+            t0 = time.perf_counter()
+            host_centroids = kmh.train(Xhost)
+            host_pointers["train_s_end_to_end"] = round(time.perf_counter() - t0, 4)
+            host_pointers["train_equals_resident"] = bool(np.array_equal(host_centroids, centroids))
+            kmh.close()
+        del Xhost
+
     # ---- CPU baseline: the oracle on a bounded prefix of the same points ----
     cpu = None
     if not args.no_cpu:
@@ -229,6 +253,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "train": train,
+        "host_pointers": host_pointers,
     }
     print(json.dumps(out))
     km.close()
