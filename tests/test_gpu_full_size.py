@@ -1,6 +1,7 @@
 """The BASELINE workloads at their real sizes, checked through size-independent properties and
 sampled exact comparisons (the CPU oracle cannot run these sizes in test time; it arbitrates samples).
 
+C1  flat Train + Assign        n=100,000    d=768  k=1,000    (the one size the CPU oracle runs in full: whole runs compared)
 C2  flat Train + Assign        n=1,000,000  d=1024 k=10,000
 C3  Assign only                n=10,000,000 d=1024 k=10,000   (41 GB of points resident in HBM)
 C4  hierarchical Train+Assign  n=10,000,000 d=1024 k=65,536
@@ -38,6 +39,44 @@ def _check_assign_sample(oracle, ids, rows, centroids, assign):
     tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
     got = assign[ids]
     assert np.all((got == bi) | tie), f"{np.sum((got != bi) & ~tie)} sampled points differ from exact brute force"
+
+
+def test_c1_flat_train_and_assign_whole_run_against_the_oracle(capi, ctx, oracle):
+    """n = 100,000, d = 768, k = 1,000, 25 iterations: 1,000 centres ~ N(0, I), point = centre + 0.3 N(0, I), rows
+    L2-normalised.  The oracle runs the whole configuration in seconds, so the two runs are compared iteration by
+    iteration: same control flow (iteration kinds, d' schedule, split counts), WCSS within 1e-3 (1e-4 before the first
+    split-induced near tie), not-pruned fraction within 1 %, final centroids within 1e-2 relative L2, <= 0.1 % of the
+    training assignments different, Assign equal to fp64 brute force except on near ties."""
+    n, d, k, iters = 100_000, 768, 1_000, 25
+    g = np.random.default_rng(1)
+    centres = g.standard_normal((k, d)).astype(np.float32)
+    X = centres[g.integers(0, k, n)] + 0.3 * g.standard_normal((n, d)).astype(np.float32)
+    X = np.ascontiguousarray(X / np.linalg.norm(X, axis=1, keepdims=True), dtype=np.float32)
+    cfg = dict(iters=iters, sampling_fraction=1.0, early_termination=0, seed=42, suppress_warnings=1)
+    km, ok = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    C, OC = km.train(X), ok.train(X)
+    gs, os_ = km.stats(), ok.stats()
+    assert len(gs) == len(os_) == iters
+    for a, b in zip(gs, os_):
+        assert (a.iteration, bool(a.is_gemm_only), a.partial_d, a.split) == \
+               (b.iteration, bool(b.is_gemm_only), b.partial_d, b.split)
+        assert abs(a.objective - b.objective_f64) <= 1e-3 * b.objective_f64
+        if not a.is_gemm_only:
+            assert abs(a.not_pruned_pct - b.not_pruned_pct) <= 1e-2 * b.not_pruned_pct + 1e-6
+    for a, b in zip(gs[:2], os_[:2]):
+        assert abs(a.objective - b.objective_f64) <= 1e-4 * b.objective_f64
+    assert gs[0].is_gemm_only and not any(s.is_gemm_only for s in gs[1:])
+    assert all(gs[i].objective <= gs[i - 1].objective * 1.01 for i in range(1, iters))
+    num = np.linalg.norm(C.astype(np.float64) - OC.astype(np.float64))
+    assert num / np.linalg.norm(OC.astype(np.float64)) <= 1e-2
+    _, oa, _, _ = ok.state()
+    assert np.mean(km.assignments(n) != oa) <= 1e-3
+    a1 = km.assign(X, C)
+    ids = np.sort(g.choice(n, 20000, replace=False))
+    _check_assign_sample(oracle, ids, X[ids], C, a1)
+    assert np.mean(a1 != ok.assign(X, C)) <= 1e-4
+    assert np.mean(km.assign_training_points(X, C) == a1) >= 0.98  # test_assign.cpp:118-155
+    km.close()
 
 
 def test_c2_flat_train_and_assign_full_size(capi, ctx, oracle):
