@@ -54,6 +54,13 @@ struct skm_kmeans {
     skmeans::SuperKMeans<>* base() { return hier ? static_cast<skmeans::SuperKMeans<>*>(hier.get()) : flat.get(); }
 };
 
+// Points the model's centroid download at the caller's buffer for the duration of one Train call.
+struct SinkScope {
+    skmeans::SuperKMeans<>* model;
+    SinkScope(skmeans::SuperKMeans<>* m, float* sink) : model(m) { model->output_sink = sink; }
+    ~SinkScope() { model->output_sink = nullptr; }
+};
+
 #define SKM_API_GUARD(body)                                                                        \
     try {                                                                                          \
         body;                                                                                      \
@@ -132,7 +139,7 @@ int skm_kmeans_train(skm_kmeans* km, const float* h_data, size_t n, const float*
                      float* h_out_centroids) {
     if (!km || !h_data || !h_out_centroids) return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_train: null argument");
     SKM_API_GUARD({
-        km->base()->output_sink = h_out_centroids;  // centroids are downloaded straight into the caller's buffer
+        SinkScope sink(km->base(), h_out_centroids);  // centroids are downloaded straight into the caller's buffer
         if (km->hier) km->hier->Train(h_data, n, h_queries, n_queries); else km->flat->Train(h_data, n, h_queries, n_queries);
         km->n_trained = n;
     });
@@ -143,7 +150,7 @@ int skm_kmeans_train_device(skm_kmeans* km, const float* d_data, size_t n, const
     if (!km || !d_data || !h_out_centroids)
         return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_train_device: null argument");
     SKM_API_GUARD({
-        km->base()->output_sink = h_out_centroids;
+        SinkScope sink(km->base(), h_out_centroids);
         if (km->hier) km->hier->TrainDevice(d_data, n, d_queries, n_queries);
         else km->flat->TrainDevice(d_data, n, d_queries, n_queries);
         km->n_trained = n;
