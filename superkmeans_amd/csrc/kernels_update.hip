@@ -9,6 +9,9 @@
 #include "skm_internal.h"
 
 #include <algorithm>
+#include <cstring>
+#include <unordered_map>
+#include <vector>
 
 namespace skm {
 
@@ -146,71 +149,87 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     }
 }
 
-// `groups` workgroups per centroid, each owning a contiguous range of columns (thread t of a group owns
-// columns 4t..4t+3 of that range).  Rows of the segment are visited in ascending point id, so the sum of every
-// column is accumulated in the reference's order whatever the number of groups; `UNROLL` independent row
-// loads are kept in flight per thread.  With many centroids one group per centroid fills the chip; with few,
-// long segments (mesoclustering: 256 centroids over 10 M points) the columns are spread over several
-// workgroups and more rows are kept in flight.
-template <bool VEC, int UNROLL>
-__global__ __launch_bounds__(256) void segment_sum_kernel(
+// Fallback for rows that cannot be read as aligned float4 (d not a multiple of 4, or an unaligned base): one
+// workgroup per centroid, one column per thread, rows in ascending point id.
+__global__ __launch_bounds__(256) void segment_sum_columns_kernel(
+    const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
+    const uint32_t* __restrict__ offsets, float* __restrict__ sums
+) {
+    const uint32_t c = blockIdx.x;
+    const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
+    float* out = sums + (size_t) c * d;
+    for (size_t t = threadIdx.x; t < d; t += blockDim.x) {
+        float acc = 0.0f;
+        for (uint32_t j = j0; j < j1; ++j) acc += x[(size_t) sorted_ids[j] * d + t];
+        out[t] = acc;
+    }
+}
+
+// Sums of the rows of every centroid's segment, in ascending point id (the reference's order of additions), so the
+// additions of one column are a chain and the time of a launch is the walk of the longest segment: hundreds of rows
+// with many centroids, tens of thousands in a mesoclustering.  One wavefront owns 64 * W consecutive columns of
+// one centroid (W = 4, 2 or 1 floats per lane: the widest that still gives every SIMD a couple of wavefronts),
+// keeps a ring of ROWS row loads in flight (a slot is requested again as soon as its row has been added) and keeps
+// the per-row work on the chain to two lane reads, the load and the add.  Requests past the end of the segment are
+// clamped to its last row so that no load sits under a condition.
+template <int W, int ROWS>
+__global__ __launch_bounds__(64) void segment_sum_deep_kernel(
     const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
     const uint32_t* __restrict__ offsets, float* __restrict__ sums, uint32_t groups
 ) {
+    static_assert(ROWS <= 64, "lane u prepares the address of row u of a batch");
+    typedef float vec_t __attribute__((ext_vector_type(W)));
     const uint32_t c = blockIdx.x / groups, g = blockIdx.x % groups;
     const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
-    float* out = sums + (size_t) c * d;
-    if (VEC) {
-        const size_t d4 = d / 4;
-        const size_t per = (d4 + groups - 1) / groups;
-        const size_t t_end = (g + 1) * per < d4 ? (g + 1) * per : d4;
-        for (size_t t = g * per + threadIdx.x; t < t_end; t += blockDim.x) {
-            float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-            uint32_t j = j0;
-            for (; j + UNROLL <= j1; j += UNROLL) {
-                float4 v[UNROLL];
+    const size_t t = (size_t) g * 64 + threadIdx.x;  // column group of this lane
+    const size_t n_groups = d / W;
+    const size_t t_load = t < n_groups ? t : n_groups - 1;  // lanes past the last column load it again and store nothing
+    vec_t acc = 0.0f;
+    if (j1 > j0) {
+        const size_t last = j1 - 1;
+        // Row addresses of a batch are prepared by the lanes in parallel (lane u: one coalesced id load and one
+        // 64-bit multiply-add for row u) and read from that lane's registers when the row is requested, which
+        // leaves two lane reads, the load and the add per row on the chain.
+        const auto batch_ids = [&](const size_t from) {
+            const size_t pos = from + threadIdx.x;
+            return sorted_ids[pos <= last ? pos : last];
+        };
+        const auto address_of = [&](const uint32_t id) { return reinterpret_cast<uint64_t>(x + (size_t) id * d); };
+        const auto row = [&](const uint64_t addresses, const int u) {
+            const uint32_t lo = __builtin_amdgcn_readlane((uint32_t) addresses, u);
+            const uint32_t hi = __builtin_amdgcn_readlane((uint32_t) (addresses >> 32), u);
+            // an address built from integers is "flat" unless it says that it is global memory; flat loads would
+            // make every wait a wait for all loads
+            typedef const vec_t __attribute__((address_space(1))) * global_row_t;
+            return reinterpret_cast<global_row_t>(((uint64_t) hi << 32) | lo)[t_load];
+        };
+        vec_t ring[ROWS];
+        uint64_t addresses = address_of(batch_ids(j0));
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u)
-                    v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
+        for (int u = 0; u < ROWS; ++u) ring[u] = row(addresses, u);
+        addresses = address_of(batch_ids((size_t) j0 + ROWS));
+        size_t j = j0;
+        for (; j + ROWS <= j1; j += ROWS) {
+            const uint32_t ids_after = batch_ids(j + 2 * ROWS);
+            __builtin_amdgcn_sched_barrier(0);
+            // every slot is added and at once requested again for the row ROWS further on: ROWS - 1 loads stay in flight
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    acc.x += v[u].x;
-                    acc.y += v[u].y;
-                    acc.z += v[u].z;
-                    acc.w += v[u].w;
-                }
+            for (int u = 0; u < ROWS; ++u) {
+                acc += ring[u];
+                ring[u] = row(addresses, u);
+                __builtin_amdgcn_sched_barrier(0);  // keeps the request next to the add instead of after all adds
             }
-            for (; j + 4 <= j1; j += 4) {
-                float4 v[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    v[u] = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j + u] * d)[t];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    acc.x += v[u].x;
-                    acc.y += v[u].y;
-                    acc.z += v[u].z;
-                    acc.w += v[u].w;
-                }
-            }
-            for (; j < j1; ++j) {
-                const float4 v = reinterpret_cast<const float4*>(x + (size_t) sorted_ids[j] * d)[t];
-                acc.x += v.x;
-                acc.y += v.y;
-                acc.z += v.z;
-                acc.w += v.w;
-            }
-            reinterpret_cast<float4*>(out)[t] = acc;
+            addresses = address_of(ids_after);
+            // The addresses are finished here, at the end of the pass that requested their ids (the ids are
+            // ROWS requests old by now).  Left to itself the compiler carries the ids into the next pass and
+            // computes there, where it must wait for every load in flight.
+            asm volatile("" : "+v"(addresses));
         }
-    } else {
-        const size_t per = (d + groups - 1) / groups;
-        const size_t t_end = (g + 1) * per < d ? (g + 1) * per : d;
-        for (size_t t = g * per + threadIdx.x; t < t_end; t += blockDim.x) {
-            float acc = 0.0f;
-            for (uint32_t j = j0; j < j1; ++j) acc += x[(size_t) sorted_ids[j] * d + t];
-            out[t] = acc;
-        }
+#pragma unroll
+        for (int u = 0; u < ROWS; ++u)
+            if (j + u < j1) acc += ring[u];
     }
+    if (t < n_groups) reinterpret_cast<vec_t*>(sums + (size_t) c * d)[t] = acc;
 }
 
 __global__ __launch_bounds__(256) void scale_by_size_kernel(
@@ -237,35 +256,34 @@ __global__ __launch_bounds__(256) void normalize_rows_kernel(float* __restrict__
     for (size_t t = lane; t < d; t += 64) p[t] *= inv;
 }
 
-// Applies the row edits of SplitClusters one after the other (later edits see earlier ones).
-__global__ __launch_bounds__(256) void edit_rows_kernel(float* __restrict__ c, size_t d, const uint32_t* __restrict__ ops, size_t n_ops) {
+// Applies row edits of SplitClusters, one workgroup per edit.  The edits of one launch touch disjoint rows (or only
+// read a common one); the host orders edits that depend on each other into successive launches.
+__global__ __launch_bounds__(256) void edit_rows_kernel(float* __restrict__ c, size_t d, const uint32_t* __restrict__ ops) {
     const float eps = 1.0f / 1024.0f;
-    for (size_t o = 0; o < n_ops; ++o) {
-        const uint32_t kind = ops[4 * o], dst = ops[4 * o + 1], src = ops[4 * o + 2];
-        const float w = __uint_as_float(ops[4 * o + 3]);
-        float* pd = c + (size_t) dst * d;
-        float* ps = c + (size_t) src * d;
-        if (kind == 0) {
-            for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
-                const float v = ps[j];
-                if (j % 2 == 0) {
-                    pd[j] = v * (1 + eps);
-                    ps[j] = v * (1 - eps);
-                } else {
-                    pd[j] = v * (1 - eps);
-                    ps[j] = v * (1 + eps);
-                }
-            }
-        } else {
-            for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
-                float val = 0.0f;
-                val += w * pd[j];
-                val += 1.0f * ps[j];
-                val /= (w + 1.0f);
-                pd[j] = val;
+    const size_t o = blockIdx.x;
+    const uint32_t kind = ops[4 * o], dst = ops[4 * o + 1], src = ops[4 * o + 2];
+    const float w = __uint_as_float(ops[4 * o + 3]);
+    float* pd = c + (size_t) dst * d;
+    float* ps = c + (size_t) src * d;
+    if (kind == 0) {
+        for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
+            const float v = ps[j];
+            if (j % 2 == 0) {
+                pd[j] = v * (1 + eps);
+                ps[j] = v * (1 - eps);
+            } else {
+                pd[j] = v * (1 - eps);
+                ps[j] = v * (1 + eps);
             }
         }
-        __syncthreads();
+    } else {
+        for (size_t j = threadIdx.x; j < d; j += blockDim.x) {
+            float val = 0.0f;
+            val += w * pd[j];
+            val += 1.0f * ps[j];
+            val /= (w + 1.0f);
+            pd[j] = val;
+        }
     }
 }
 
@@ -400,22 +418,23 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     SKM_HIP_TRY(hipGetLastError());
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
-    const size_t lanes = vec ? d / 4 : d;
-    // Few centroids: spread the columns of a centroid over several workgroups of at least one wavefront until
-    // about 2,048 workgroups are in flight, and keep more rows in flight when segments are long on average.
-    size_t groups = 1;
-    while (k * groups < 2048 && lanes / (groups * 2) >= 64) groups *= 2;
-    const size_t per = (lanes + groups - 1) / groups;
-    unsigned threads = (unsigned) std::min<size_t>(256, ((per + 63) / 64) * 64);
-    dim3 grid((unsigned) (k * groups));
-    const bool long_segments = n / k >= 1024;
-    if (vec && long_segments)
-        hipLaunchKernelGGL((segment_sum_kernel<true, 32>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
-    else if (vec)
-        hipLaunchKernelGGL((segment_sum_kernel<true, 16>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
-    else
-        hipLaunchKernelGGL((segment_sum_kernel<false, 16>), grid, dim3(threads), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
-    return check_hip(hipGetLastError(), "segment_sum_kernel launch");
+    if (vec) {
+        // widest lanes that still give about 2,048 wavefronts
+        int w = 4;
+        while (w > 1 && k * ((d / w + 63) / 64) < 2048) w /= 2;
+        const size_t groups = (d / w + 63) / 64;
+        SKM_REQUIRE(k * groups <= 0x7fffffffULL, "k * d too large for one launch");
+        dim3 grid((unsigned) (k * groups));
+        if (w == 4)
+            hipLaunchKernelGGL((segment_sum_deep_kernel<4, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+        else if (w == 2)
+            hipLaunchKernelGGL((segment_sum_deep_kernel<2, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+        else
+            hipLaunchKernelGGL((segment_sum_deep_kernel<1, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+    } else {
+        hipLaunchKernelGGL(segment_sum_columns_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+    }
+    return check_hip(hipGetLastError(), "segment sum launch");
 }
 
 int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d) {
@@ -438,12 +457,52 @@ int skm_edit_rows(skm_ctx* ctx, float* d_c, size_t d, const uint32_t* h_ops, siz
     SKM_REQUIRE(ctx && d_c, "null argument");
     if (n_ops == 0) return SKM_OK;
     SKM_REQUIRE(h_ops, "null ops");
+    SKM_REQUIRE(n_ops <= 0x7fffffffu, "too many edits");
+    // Later edits see earlier ones.  Edits that touch disjoint rows commute, so every edit gets the earliest
+    // round in which all edits it depends on are done (an earlier edit wrote a row it reads or writes, or read a
+    // row it writes), and the rounds run one launch after the other with one workgroup per edit.
+    std::unordered_map<uint32_t, int> last_write, last_read;
+    std::vector<int> round(n_ops);
+    int n_rounds = 0;
+    const auto seen = [](const std::unordered_map<uint32_t, int>& m, const uint32_t row) {
+        const auto it = m.find(row);
+        return it == m.end() ? -1 : it->second;
+    };
+    for (size_t o = 0; o < n_ops; ++o) {
+        const uint32_t kind = h_ops[4 * o], dst = h_ops[4 * o + 1], src = h_ops[4 * o + 2];
+        SKM_REQUIRE(kind <= 1, "unknown edit kind");
+        // kind 0 writes both rows, kind 1 writes dst and reads both
+        int r = std::max({seen(last_write, dst), seen(last_write, src), seen(last_read, dst)});
+        if (kind == 0) r = std::max(r, seen(last_read, src));
+        r += 1;
+        round[o] = r;
+        n_rounds = std::max(n_rounds, r + 1);
+        last_write[dst] = r;
+        if (kind == 0) {
+            last_write[src] = r;
+        } else {
+            last_read[src] = std::max(seen(last_read, src), r);
+        }
+    }
+    std::vector<uint32_t> ordered(n_ops * 4);
+    std::vector<size_t> first(n_rounds + 1, 0);
+    for (size_t o = 0; o < n_ops; ++o) first[round[o] + 1]++;
+    for (int r = 0; r < n_rounds; ++r) first[r + 1] += first[r];
+    {
+        std::vector<size_t> cursor(first.begin(), first.end() - 1);
+        for (size_t o = 0; o < n_ops; ++o) std::memcpy(&ordered[4 * cursor[round[o]]++], h_ops + 4 * o, 4 * sizeof(uint32_t));
+    }
     void* ws = nullptr;
     SKM_TRY(workspace(ctx, 2, n_ops * 4 * sizeof(uint32_t), &ws));
-    SKM_HIP_TRY(hipMemcpyAsync(ws, h_ops, n_ops * 4 * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
-    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));  // h_ops is caller memory: do not outlive the call
-    hipLaunchKernelGGL(edit_rows_kernel, dim3(1), dim3(256), 0, ctx->stream, d_c, d, (const uint32_t*) ws, n_ops);
-    return check_hip(hipGetLastError(), "edit_rows_kernel launch");
+    SKM_HIP_TRY(hipMemcpyAsync(ws, ordered.data(), n_ops * 4 * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));  // `ordered` is released on return
+    for (int r = 0; r < n_rounds; ++r) {
+        const size_t count = first[r + 1] - first[r];
+        hipLaunchKernelGGL(edit_rows_kernel, dim3((unsigned) count), dim3(256), 0, ctx->stream, d_c, d,
+                           (const uint32_t*) ws + 4 * first[r]);
+        SKM_TRY(check_hip(hipGetLastError(), "edit_rows_kernel launch"));
+    }
+    return SKM_OK;
 }
 
 int skm_wcss(skm_ctx* ctx, const float* d_dist, size_t n, double* h_out_cost) {

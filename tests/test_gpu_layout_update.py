@@ -169,6 +169,35 @@ def test_edit_rows_matches_split_clusters(capi, ctx, oracle):
     dC.free()
 
 
+@pytest.mark.parametrize("k,n_ops,seed", [(6, 300, 0), (40, 500, 1), (3000, 2000, 2)])
+def test_edit_rows_dependent_edits_apply_in_order(capi, ctx, k, n_ops, seed):
+    """Edits run concurrently where they touch disjoint rows and in order where one reads or writes a row another
+    wrote (or writes a row another read): any sequence must give what one-after-the-other application gives, bit for
+    bit.  Few rows and many edits make long dependency chains; many rows make wide rounds."""
+    g = np.random.default_rng(seed)
+    d = 70
+    C = g.standard_normal((k, d)).astype(np.float32)
+    ops = np.zeros((n_ops, 4), dtype=np.uint32)
+    exp = C.copy()
+    eps = np.float32(1.0 / 1024.0)
+    even = np.arange(d) % 2 == 0
+    for o in range(n_ops):
+        kind = int(g.integers(0, 2))
+        dst, src = (int(v) for v in g.choice(k, 2, replace=False))
+        w = np.float32(g.integers(1, 8))
+        ops[o] = (kind, dst, src, w.view(np.uint32))
+        if kind == 0:
+            v = exp[src].copy()
+            exp[dst] = np.where(even, v * (np.float32(1) + eps), v * (np.float32(1) - eps))
+            exp[src] = np.where(even, v * (np.float32(1) - eps), v * (np.float32(1) + eps))
+        else:
+            exp[dst] = (np.float32(0) + w * exp[dst] + np.float32(1) * exp[src]) / (w + np.float32(1))
+    dC = ctx.array(C)
+    capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, ops.ctypes.data, n_ops))
+    assert np.array_equal(dC.download(), exp)
+    dC.free()
+
+
 def test_edit_rows_balancing_and_normalize(capi, ctx):
     g = np.random.default_rng(10)
     C = g.standard_normal((5, 96)).astype(np.float32)
