@@ -288,7 +288,25 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
     const float* cp = c + (int64_t) idx[p] * d;
     float s = 0.0f;
     if (VEC) {
-        for (int t = lane * 4; t < d; t += 256) {
+        // four strides of 256 columns are requested together (eight loads in flight), then added in column order
+        int t = lane * 4;
+        for (; t + 768 < d; t += 1024) {
+            float4 xv[4], cv[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                xv[u] = *reinterpret_cast<const float4*>(xq + t + 256 * u);
+                cv[u] = *reinterpret_cast<const float4*>(cp + t + 256 * u);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                float e;
+                e = cv[u].x - xv[u].x; s += e * e;
+                e = cv[u].y - xv[u].y; s += e * e;
+                e = cv[u].z - xv[u].z; s += e * e;
+                e = cv[u].w - xv[u].w; s += e * e;
+            }
+        }
+        for (; t < d; t += 256) {
             const float4 xv = *reinterpret_cast<const float4*>(xq + t);
             const float4 cv = *reinterpret_cast<const float4*>(cp + t);
             float e;
