@@ -155,14 +155,16 @@ class ADSamplingPruner {
         InitializeRatios();
     }
 
-    // out = vectors . Q^T, both device-resident (n x d).
-    void Rotate(const float* d_vectors, float* d_out, const size_t n) const {
-        hip::Check(skm_rotate(ctx_, d_vectors, n, num_dimensions, d_q_.get(), d_out));
+    // out = vectors . Q^T, both device-resident (n x d), queued on `on` (objects that share these tables each
+    // rotate on their own context).
+    void Rotate(skm_ctx* on, const float* d_vectors, float* d_out, const size_t n) const {
+        hip::Check(skm_rotate(on, d_vectors, n, num_dimensions, d_q_.get(), d_out));
     }
     // out = rotated . Q, both device-resident.
-    void Unrotate(const float* d_rotated, float* d_out, const size_t n) const {
-        hip::Check(skm_unrotate(ctx_, d_rotated, n, num_dimensions, d_qt_.get(), d_out));
+    void Unrotate(skm_ctx* on, const float* d_rotated, float* d_out, const size_t n) const {
+        hip::Check(skm_unrotate(on, d_rotated, n, num_dimensions, d_qt_.get(), d_out));
     }
+    float Epsilon0() const { return epsilon0; }
 
     const float* DeviceRatios() const { return d_ratios_.get(); }
     const std::vector<float>& HostMatrix() const { return matrix_; }

@@ -22,6 +22,7 @@
 #include <numeric>
 #include <random>
 #include <sstream>
+#include <thread>
 #include <vector>
 
 #include "superkmeans/common.h"
@@ -225,16 +226,17 @@ class SuperKMeans {
         }
         partial_d = std::max<uint32_t>(MIN_PARTIAL_D, vertical_d / 2);
 
-        // Rotated copy of the caller's vectors (or the vectors themselves when already rotated).
-        dbuf<float> d_rot(ctx, n_vectors * d);
+        // The caller's vectors go to the device in slabs; every slab is rotated while the next one is copied
+        // (already rotated vectors are used as they arrive).  The raw copy is kept for the seeding below.
+        dbuf<float> d_rot(ctx, n_vectors * d), d_raw;
+        if (!config.data_already_rotated) d_raw.Reset(ctx, n_vectors * d);
+        dbuf<float>& landing = config.data_already_rotated ? d_rot : d_raw;
         {
-            if (config.data_already_rotated) {
-                d_rot.Upload(vectors, n_vectors * d);
-            } else {
-                dbuf<float> d_raw(ctx, n_vectors * d);
-                d_raw.Upload(vectors, n_vectors * d);
-                pruner->Rotate(d_raw.get(), d_rot.get(), n_vectors);
-                hip::Check(skm_sync(ctx));
+            const size_t slab = UploadSlabRows();
+            for (size_t r0 = 0; r0 < n_vectors; r0 += slab) {
+                const size_t m = std::min(slab, n_vectors - r0);
+                landing.UploadOverlapped(vectors + r0 * d, m * d, r0 * d);
+                if (!config.data_already_rotated) pruner->Rotate(ctx, d_raw.get() + r0 * d, d_rot.get() + r0 * d, m);
             }
         }
         // Final centroids: horizontal_centroids / centroids (PDX) / partial_horizontal_centroids were
@@ -264,10 +266,28 @@ class SuperKMeans {
             tmp_config.seed = config.seed;
             tmp_config.angular = config.angular;
             tmp_config.data_already_rotated = config.data_already_rotated;
+            tmp_config.dct_rotation = config.dct_rotation;
             auto new_n_centroids = static_cast<size_t>(std::sqrt(n_centroids));
-            SuperKMeans tmp_kmeans(new_n_centroids, d, tmp_config);
+            // Same dimensionality and seed as this object: the rotation matrix and ratios would come out the same,
+            // so the tables are shared instead of being factorised again on the host (the hierarchical variant
+            // holds tables with another epsilon and builds fresh ones, as the reference does).
+            std::unique_ptr<SuperKMeans> tmp_owner(
+                pruner->Epsilon0() == PRUNER_INITIAL_THRESHOLD
+                    ? new SuperKMeans(new_n_centroids, d, tmp_config, pruner)
+                    : new SuperKMeans(new_n_centroids, d, tmp_config));
+            SuperKMeans& tmp_kmeans = *tmp_owner;
             auto meso_centroids = tmp_kmeans.Train(centroids, n_centroids);
-            auto meso_assignments = tmp_kmeans.Assign(vectors, meso_centroids.data(), n_vectors, new_n_centroids);
+            // Nearest meso-centroid of every vector, on the copy that is already on the device.
+            hip::Check(skm_sync(ctx));
+            std::vector<uint32_t> meso_assignments(n_vectors);
+            {
+                skm_ctx* tctx = tmp_kmeans.GetContext();
+                dbuf<float> d_meso(tctx, new_n_centroids * d);
+                d_meso.Upload(meso_centroids.data(), new_n_centroids * d);
+                dbuf<uint32_t> d_meso_assignments(tctx, n_vectors);
+                tmp_kmeans.AssignDevice(landing.get(), d_meso.get(), n_vectors, new_n_centroids, d_meso_assignments.get());
+                d_meso_assignments.Download(meso_assignments.data(), n_vectors);
+            }
             auto centroids_to_meso = tmp_kmeans.Assign(centroids, meso_centroids.data(), n_centroids, new_n_centroids);
             g_n_threads = n_threads;
             std::vector<uint32_t> meso_to_original(new_n_centroids, 0);
@@ -735,7 +755,7 @@ class SuperKMeans {
 
     void RotateOrCopy(const float* d_in, float* d_out, const size_t n_vectors, const bool rotate) {
         if (rotate) {
-            pruner->Rotate(d_in, d_out, n_vectors);
+            pruner->Rotate(ctx, d_in, d_out, n_vectors);
         } else {
             hip::Check(skm_copy(ctx, d_out, d_in, sizeof(float) * n_vectors * d));
         }
@@ -809,7 +829,7 @@ class SuperKMeans {
         }
         if (should_unrotate) {
             dbuf<float> unrotated(ctx, n_clusters * d);
-            pruner->Unrotate(horizontal_centroids.get(), unrotated.get(), n_clusters);
+            pruner->Unrotate(ctx, horizontal_centroids.get(), unrotated.get(), n_clusters);
             unrotated.Download(dst, n_clusters * d);
         } else {
             horizontal_centroids.Download(dst, n_clusters * d);
@@ -845,7 +865,7 @@ class SuperKMeans {
             for (size_t r0 = 0; r0 < n_samples_; r0 += slab) {
                 const size_t m = std::min(slab, n_samples_ - r0);
                 landing.UploadOverlapped(data + r0 * d, m * d, r0 * d);
-                if (rotate) pruner->Rotate(raw.get() + r0 * d, training_data.get() + r0 * d, m);
+                if (rotate) pruner->Rotate(ctx, raw.get() + r0 * d, training_data.get() + r0 * d, m);
                 if (after_slab) after_slab(training_data.get() + r0 * d, r0, m);
             }
             if (rotate) hip::Check(skm_sync(ctx));  // `raw` is released on return
@@ -870,8 +890,7 @@ class SuperKMeans {
             std::vector<float> host(std::min(slab, n_samples_) * d);
             for (size_t i0 = 0; i0 < n_samples_; i0 += slab) {
                 const size_t m = std::min(slab, n_samples_ - i0);
-                for (size_t i = 0; i < m; ++i)
-                    std::memcpy(&host[i * d], data + sampled_indices[i0 + i] * d, sizeof(float) * d);
+                GatherHostRows(host.data(), data, sampled_indices.get() + i0, m);
                 staged.Upload(host.data(), m * d, i0 * d);
             }
             d_raw = staged.get();
@@ -881,9 +900,28 @@ class SuperKMeans {
             return training_data.get();
         }
         training_data.Reset(ctx, n_samples_ * d);
-        pruner->Rotate(d_raw, training_data.get(), n_samples_);
+        pruner->Rotate(ctx, d_raw, training_data.get(), n_samples_);
         if (staged.get() != nullptr) hip::Check(skm_sync(ctx));  // `staged` is released on return
         return training_data.get();
+    }
+
+    // dst[i] = data[rows[i]] for i < count.  The rows are scattered over a matrix of gigabytes, so the copy is
+    // bound by memory latency: a few host threads split the range.
+    void GatherHostRows(float* dst, const vector_value_t* data, const size_t* rows, const size_t count) const {
+        const size_t row_bytes = sizeof(float) * d;
+        size_t workers = std::min<size_t>(std::max(1u, std::thread::hardware_concurrency()), 8);
+        workers = std::min(workers, std::max<size_t>(1, count * row_bytes >> 22));  // at least 4 MiB per thread
+        const auto copy_range = [&](const size_t begin, const size_t end) {
+            for (size_t i = begin; i < end; ++i) std::memcpy(dst + i * d, data + rows[i] * d, row_bytes);
+        };
+        if (workers <= 1) {
+            copy_range(0, count);
+            return;
+        }
+        std::vector<std::thread> pool;
+        for (size_t w = 1; w < workers; ++w) pool.emplace_back(copy_range, count * w / workers, count * (w + 1) / workers);
+        copy_range(0, count / workers);
+        for (auto& t : pool) t.join();
     }
 
     // Copies the device assignments / distances of the training points to the public host members.
