@@ -173,6 +173,14 @@ int skm_recall_hits(skm_ctx* ctx, const uint32_t* d_gt, const uint32_t* d_promis
                     const uint32_t* d_assignments, size_t n_assignments, size_t n_queries,
                     size_t objective_k, size_t explore, uint32_t* h_out_hits);
 
+/* Orthogonal factor Q = H_0 H_1 ... H_{d-1} of the Householder QR of the d x d matrix h_a (row-major, double), as
+ * float, into h_out_q.  The reference obtains its rotation matrix this way on the CPU (pdx/adsampling.h:76-85,
+ * Eigen::HouseholderQR of a Gaussian matrix).  Evaluated on the device in double with the operations and the
+ * summation order of skmeans::detail::OrthogonalFactor (superkmeans/pdx/adsampling.h), whose result it equals
+ * bit for bit; d <= SKM_HOUSEHOLDER_Q_MAX_D (a workgroup keeps all rows of eight columns in LDS). */
+#define SKM_HOUSEHOLDER_Q_MAX_D 2272
+int skm_householder_q(skm_ctx* ctx, const double* h_a, size_t d, float* h_out_q);
+
 /* Benchmark / test utility: seeded Gaussian-mixture rows generated in device memory.  Row i (logical
  * index row_offset + local row) is  s_j * (center_sigma * g(center_seed, u_i, j) + noise_sigma *
  * g(point_seed, i, j)),  s_j = (j + 1)^(-decay_exponent),  u_i = hash(i) mod n_centers (n_centers == 0:

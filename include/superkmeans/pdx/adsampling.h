@@ -118,6 +118,8 @@ class ADSamplingPruner {
   public:
     uint32_t num_dimensions;
     std::vector<float> ratios;  // ratios[v]: factor applied to the best distance after v dimensions
+    // Below this the factorisation is a few milliseconds on the host and the device's launches cost as much.
+    static constexpr size_t DEVICE_FACTORISATION_MIN_D = 384;
 
     // Draws d*d N(0,1) values row by row from std::mt19937(seed) through
     // std::normal_distribution<float> (the reference's sequence, pdx/adsampling.h:76-82) and keeps
@@ -135,7 +137,14 @@ class ADSamplingPruner {
             std::normal_distribution<float> dist(0.0f, 1.0f);
             std::vector<double> a(d * d);
             for (size_t i = 0; i < d * d; ++i) a[i] = dist(gen);
-            matrix_ = detail::OrthogonalFactor(std::move(a), d);
+            if (d >= DEVICE_FACTORISATION_MIN_D && d <= SKM_HOUSEHOLDER_Q_MAX_D) {
+                // same operations in the same order on the device: the matrix is the host routine's, bit for bit,
+                // in a fraction of the time at d = 1024
+                matrix_.resize(d * d);
+                hip::Check(skm_householder_q(ctx_, a.data(), d, matrix_.data()));
+            } else {
+                matrix_ = detail::OrthogonalFactor(std::move(a), d);
+            }
         }
         d_q_.Reset(ctx_, d * d);
         d_qt_.Reset(ctx_, d * d);

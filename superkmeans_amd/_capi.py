@@ -30,6 +30,7 @@ _PROTOTYPES = {
     "skm_free": (c_int, [c_void_p, c_void_p]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_upload_overlapped": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "skm_householder_q": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "skm_download": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_fill_u32": (c_int, [c_void_p, c_void_p, c_uint32, c_size_t]),
