@@ -51,6 +51,9 @@ struct GemmShape {
 };
 using GemmSmall = GemmShape<2, 2, 2, 2, 2>;
 using GemmBig = GemmShape<2, 4, 4, 2, 1>;
+// 32 x 128: a handful of M rows against all N rows, bound by the loads of the N operand.  Used for the centroids
+// left over when k is a few rows more than a multiple of the large shape's 256.
+using GemmThin = GemmShape<1, 4, 1, 1, 2>;
 
 constexpr int GEMM_TM = GemmSmall::TM;
 constexpr int GEMM_TN = GemmSmall::TN;
@@ -62,6 +65,7 @@ struct GemmOperands {
     int M, N, K;
     int64_t lda, ldb;
     int tiles_m, tiles_n;
+    int m_base;  // added to the row indices the argmin kernel reports (a launch over rows m_base.. of a larger matrix)
 };
 
 // Accumulators of one wavefront: acc.v[mb][nb] is a 32 x 32 block.  Element r of
