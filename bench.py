@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Super K-Means assign/update hot path on one MI355X.
 
-Workload (BASELINE config 2): n = 1,000,000 points, d = 1024, k = 10,000 centroids, fp32, seeded
+Workload (the headline configuration): n = 1,000,000 points, d = 1024, k = 10,000 centroids, fp32, seeded
 Gaussian mixture of 10,000 centres with per-dimension variance decaying as 1/sqrt(j+1), rows
 L2-normalised, generated directly in HBM.
 

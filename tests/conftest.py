@@ -42,7 +42,7 @@ def ctx(capi):
 
 
 def make_blobs(n, d, k, std=0.3, seed=0, normalize=True, center_scale=1.0):
-    """Seeded isotropic Gaussian mixture (the shape of BASELINE config C1)."""
+    """Seeded isotropic Gaussian mixture (the shape of the CPU-sized benchmark configuration)."""
     g = np.random.default_rng(seed)
     centers = (center_scale * g.standard_normal((k, d))).astype(np.float32)
     a = g.integers(0, k, n)

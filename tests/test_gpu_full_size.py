@@ -1,4 +1,4 @@
-"""The BASELINE workloads at their real sizes, checked through size-independent properties and
+"""The benchmark configurations at their real sizes, checked through size-independent properties and
 sampled exact comparisons (the CPU oracle cannot run these sizes in test time; it arbitrates samples).
 
 C1  flat Train + Assign        n=100,000    d=768  k=1,000    (the one size the CPU oracle runs in full: whole runs compared)
