@@ -185,9 +185,9 @@ def main():
     roofline = {"kernel": "gemm_argmin_kernel", "bound": "mfma", "achieved": round(achieved, 2),
                 "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
                 "traffic": MEASURED_TRAFFIC_BYTES.get((n, d, k)), "avg_launch_ms": round(gemm_avg_ms, 3), "flops_per_launch": flops_per_launch}
-    if 0 < k % 256 <= 32 and k > 256:
+    if 0 < k % 256 <= 128 and k > 256:
         # the exact search is then two launches of the same kernel; avg_launch_ms is their sum
-        roofline["launches"] = (f"256x256 tiles over the first {k - k % 256} centroids + 32x128 tiles over the last "
+        roofline["launches"] = (f"256x256 tiles over the first {k - k % 256} centroids + {32 * ((k % 256 + 31) // 32)}x128 tiles over the last "
                                 f"{k % 256}")
     gpu_assign = dOut.download()
 

@@ -51,9 +51,11 @@ struct GemmShape {
 };
 using GemmSmall = GemmShape<2, 2, 2, 2, 2>;
 using GemmBig = GemmShape<2, 4, 4, 2, 1>;
-// 32 x 128: a handful of M rows against all N rows, bound by the loads of the N operand.  Used for the centroids
-// left over when k is a few rows more than a multiple of the large shape's 256.
-using GemmThin = GemmShape<1, 4, 1, 1, 2>;
+// (32 FM) x 128: a few M rows against all N rows, bound by the loads of the N operand.  Used for the centroids left
+// over when k is up to 128 rows more than a multiple of the large shape's 256.
+template <int FM>
+using GemmThin = GemmShape<1, 4, FM, 1, 2>;
+constexpr int GEMM_THIN_MAX_ROWS = 128;
 
 constexpr int GEMM_TM = GemmSmall::TM;
 constexpr int GEMM_TN = GemmSmall::TN;

@@ -274,11 +274,11 @@ static int launch_gemm_argmin_shape(skm_ctx* ctx, const float* C, int k, const f
 
 // Centroids that the large shape would compute as a nearly empty tile row (k = 10,000 is 39 rows of 256 and 16
 // centroids: 2.4 % of the launch for 0.16 % of the work) are searched by a second, thin launch instead, which costs
-// one more read of the points.  Returns how many leading centroids go to the main launch; the rest (at most one thin
-// granule) go to the thin one.
+// one more read of the points.  Returns how many leading centroids go to the main launch; the rest (at most 128, one
+// granule slot of the large shape) go to the thin one.
 int gemm_argmin_main_rows(int k, int n) {
     const int rest = k % GemmBig::TM;
-    if (rest == 0 || rest > GemmThin::WAVE_M || k - rest < GemmBig::TM) return k;
+    if (rest == 0 || rest > GEMM_THIN_MAX_ROWS || k - rest < GemmBig::TM) return k;
     return use_big_tiles(k - rest, n) ? k - rest : k;
 }
 
@@ -294,9 +294,18 @@ int launch_gemm_argmin(skm_ctx* ctx, const float* C, int k, const float* X, int 
         const int k_main = gemm_argmin_main_rows(k, n);
         SKM_TRY(launch_gemm_argmin_shape<GemmBig>(ctx, C, k_main, X, n, d, ldc, ldx, xnorm, cnorm, granule_min));
         if (k_main == k) return SKM_OK;
-        // the leftover centroids fill the granule slot that follows the main launch's (k_main is a multiple of 256)
-        return launch_gemm_argmin_shape<GemmThin>(ctx, C + (int64_t) k_main * ldc, k - k_main, X, n, d, ldc, ldx, xnorm,
-                                                  cnorm + k_main, granule_min + (int64_t) (k_main / granule) * n, k_main);
+        // the leftover centroids (at most 128) fill the granule slot that follows the main launch's (k_main is a
+        // multiple of 256); the thin shape is as tall as they need, in steps of 32 rows
+        const float* c_rest = C + (int64_t) k_main * ldc;
+        uint2* slot = granule_min + (int64_t) (k_main / granule) * n;
+        const int rest = k - k_main;
+        if (rest <= 32)
+            return launch_gemm_argmin_shape<GemmThin<1>>(ctx, c_rest, rest, X, n, d, ldc, ldx, xnorm, cnorm + k_main, slot, k_main);
+        if (rest <= 64)
+            return launch_gemm_argmin_shape<GemmThin<2>>(ctx, c_rest, rest, X, n, d, ldc, ldx, xnorm, cnorm + k_main, slot, k_main);
+        if (rest <= 96)
+            return launch_gemm_argmin_shape<GemmThin<3>>(ctx, c_rest, rest, X, n, d, ldc, ldx, xnorm, cnorm + k_main, slot, k_main);
+        return launch_gemm_argmin_shape<GemmThin<4>>(ctx, c_rest, rest, X, n, d, ldc, ldx, xnorm, cnorm + k_main, slot, k_main);
     }
     if (granule == GemmSmall::WAVE_M)
         return launch_gemm_argmin_shape<GemmSmall>(ctx, C, k, X, n, d, ldc, ldx, xnorm, cnorm, granule_min);

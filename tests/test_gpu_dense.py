@@ -73,20 +73,21 @@ def test_assign_full_clustered_data_exact_agreement(capi, ctx, oracle, blobs):
 
 
 @pytest.mark.parametrize("n,k,d", [(70001, 1250, 96), (66000, 1500, 70), (70000, 1024, 33),
-                                   (70000, 1040, 96), (66000, 1056, 70), (70001, 1029, 33), (140000, 517, 64)])
+                                   (70000, 1040, 96), (66000, 1056, 70), (70001, 1029, 33), (140000, 517, 64),
+                                   (70000, 1064, 96), (66000, 1120, 70), (70001, 1152, 33)])
 def test_assign_full_workgroup_tile_shape_never_changes_a_bit(capi, ctx, oracle, n, k, d):
     """At least 1,024 tiles of 256 x 256 select the large workgroup shape, fewer the 128 x 128 one; a k that is up to
-    32 more than a multiple of 256 (1040, 1056, 1029, 517) sends the leftover centroids through a third, thin shape
-    in a launch of their own.  All accumulate every dot product in the same order, so one call over all points and
+    128 more than a multiple of 256 (1040, 1056, 1029, 517, 1064, 1120, 1152) sends the leftover centroids through
+    thin shapes of 32 to 128 rows in a launch of their own.  All accumulate every dot product in the same order, so one call over all points and
     calls over slices of 8,192 points must return identical bits (ragged n and k, rows that are not 16-byte aligned,
     a trailing partial slice of d), and a nearest centroid among the leftover ones must be found like any other."""
     g = np.random.default_rng(n + k + d)
     X = g.standard_normal((n, d)).astype(np.float32)
     C = g.standard_normal((k, d)).astype(np.float32)
-    if k % 256 and k % 256 <= 32:
+    if k % 256 and k % 256 <= 128:
         X[::7] = C[-(np.arange(len(X[::7])) % (k % 256)) - 1] + 0.3 * X[::7]  # every 7th point sits near a leftover centroid
     gi, gd, _ = _assign_full(capi, ctx, X, C)
-    if k % 256 and k % 256 <= 32:
+    if k % 256 and k % 256 <= 128:
         assert np.mean(gi[::7] >= k - k % 256) > 0.99
     for i0 in range(0, n, 8192):
         si, sd, _ = _assign_full(capi, ctx, X[i0:i0 + 8192], C)
