@@ -64,8 +64,9 @@ int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);
 /* Upload on the context's transfer stream: work queued on the context before the call keeps running during the
  * copy, work queued after it starts when the copy is complete.  Lets Train/Assign on host pointers (reference
  * superkmeans.h:162,346 take host pointers only) compute on one slab of rows while the next one is on its way.
- * d_dst must not be in use by work queued earlier; h_src must stay unchanged until the context is synchronised
- * (skm_sync, skm_download or skm_upload). */
+ * d_dst must not be in use by work queued earlier.  A pageable h_src has been read when the call returns (the
+ * runtime stages it); pinned memory must stay unchanged until the context is synchronised (skm_sync,
+ * skm_download or skm_upload). */
 int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int skm_copy(skm_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
 int skm_fill_u32(skm_ctx* ctx, void* d_dst, uint32_t value, size_t count);

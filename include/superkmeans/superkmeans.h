@@ -395,8 +395,8 @@ class SuperKMeans {
         const bool rotate = !config.data_already_rotated;
         const float* data_to_cluster = nullptr;
         first_search_done = false;
-        if (!on_device && n_samples == n && config.iters > 0) {
-            // Host rows that are all used: they reach the device in slabs, and every slab is rotated and searched
+        if (!on_device && config.iters > 0) {
+            // Host rows (all of them, or the sampled ones): they reach the device in slabs, and every slab is rotated and searched
             // against the initial centroids (the first iteration is always exact) while the next one is on its
             // way.  The initial centroids come first for that; they are rows of the host matrix.
             GenerateCentroids(data, n_samples, n_clusters, rotate, on_device);
@@ -854,45 +854,53 @@ class SuperKMeans {
             std::shuffle(sampled_indices.get(), sampled_indices.get() + n, rng);
         }
         if (on_device && !sample && !rotate) return data;
-        if (!on_device && !sample) {
-            // All host rows in order: slab after slab on the transfer stream, each one rotated (and handed to
-            // after_slab: training rows on the device, first row, count) while the next is copied.
+        if (!on_device) {
+            // Host rows: slab after slab on the transfer stream, each one rotated (and handed to after_slab:
+            // training rows on the device, first row, count) while the next is copied.  All rows in order are
+            // copied from where they lie; sampled rows are gathered into one of two staging buffers, the next
+            // slab by a helper thread during the copy of the current one (a copy from pageable memory returns
+            // once the source has been read).
             training_data.Reset(ctx, n_samples_ * d);
             dbuf<float> raw;
             if (rotate) raw.Reset(ctx, n_samples_ * d);
             dbuf<float>& landing = rotate ? raw : training_data;
-            const size_t slab = UploadSlabRows();
-            for (size_t r0 = 0; r0 < n_samples_; r0 += slab) {
+            const size_t slab = sample ? std::max<size_t>(1, (size_t(64) << 20) / (d * sizeof(float))) : UploadSlabRows();
+            std::vector<float> host[2];
+            const auto gather = [&](const size_t which, const size_t i0) {
+                const size_t m = std::min(slab, n_samples_ - i0);
+                host[which].resize(m * d);
+                GatherHostRows(host[which].data(), data, sampled_indices.get() + i0, m);
+            };
+            if (sample) gather(0, 0);
+            size_t which = 0;
+            for (size_t r0 = 0; r0 < n_samples_; r0 += slab, which ^= 1) {
                 const size_t m = std::min(slab, n_samples_ - r0);
-                landing.UploadOverlapped(data + r0 * d, m * d, r0 * d);
-                if (rotate) pruner->Rotate(ctx, raw.get() + r0 * d, training_data.get() + r0 * d, m);
-                if (after_slab) after_slab(training_data.get() + r0 * d, r0, m);
+                std::thread ahead;
+                if (sample && r0 + slab < n_samples_) ahead = std::thread(gather, which ^ 1, r0 + slab);
+                try {
+                    landing.UploadOverlapped(sample ? host[which].data() : data + r0 * d, m * d, r0 * d);
+                    if (rotate) pruner->Rotate(ctx, raw.get() + r0 * d, training_data.get() + r0 * d, m);
+                    if (after_slab) after_slab(training_data.get() + r0 * d, r0, m);
+                } catch (...) {
+                    if (ahead.joinable()) ahead.join();
+                    throw;
+                }
+                if (ahead.joinable()) ahead.join();
             }
             if (rotate) hip::Check(skm_sync(ctx));  // `raw` is released on return
             return training_data.get();
         }
         dbuf<float> staged;  // raw rows on the device, in training order
         const float* d_raw = nullptr;
-        if (on_device && !sample) {
+        if (!sample) {
             d_raw = data;
-        } else if (on_device) {
+        } else {
             std::vector<uint64_t> rows(sampled_indices.get(), sampled_indices.get() + n_samples_);
             dbuf<uint64_t> d_rows(ctx, n_samples_);
             d_rows.Upload(rows.data(), n_samples_);
             staged.Reset(ctx, n_samples_ * d);
             hip::Check(skm_gather_rows(ctx, data, d, d_rows.get(), n_samples_, staged.get(), nullptr, nullptr));
             hip::Check(skm_sync(ctx));
-            d_raw = staged.get();
-        } else {
-            staged.Reset(ctx, n_samples_ * d);
-            // Gather on the host in slabs so the staging buffer stays small.
-            const size_t slab = std::max<size_t>(1, (size_t(64) << 20) / (d * sizeof(float)));
-            std::vector<float> host(std::min(slab, n_samples_) * d);
-            for (size_t i0 = 0; i0 < n_samples_; i0 += slab) {
-                const size_t m = std::min(slab, n_samples_ - i0);
-                GatherHostRows(host.data(), data, sampled_indices.get() + i0, m);
-                staged.Upload(host.data(), m * d, i0 * d);
-            }
             d_raw = staged.get();
         }
         if (!rotate) {

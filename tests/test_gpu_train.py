@@ -206,9 +206,14 @@ def test_host_rows_arriving_in_slabs_give_the_device_resident_result(capi, ctx):
     kr = capi.KMeans(k, d, iters=2, sampling_fraction=1.0, early_termination=0, data_already_rotated=1)
     kq = capi.KMeans(k, d, iters=2, sampling_fraction=1.0, early_termination=0, data_already_rotated=1)
     assert np.array_equal(kr.train(X), kq.train_device(dX, n))
+    # sampled rows are gathered on the host into two alternating 64 MiB buffers (five slabs here) and take the same path
+    ks = capi.KMeans(k, d, iters=3, sampling_fraction=0.5, early_termination=0)
+    kt = capi.KMeans(k, d, iters=3, sampling_fraction=0.5, early_termination=0)
+    assert np.array_equal(ks.train(X), kt.train_device(dX, n))
+    assert [(s.objective, s.shift, s.split) for s in ks.stats()] == [(s.objective, s.shift, s.split) for s in kt.stats()]
     for o in (dX, dC, dOut):
         o.free()
-    km.close(), kh.close(), kr.close(), kq.close()
+    km.close(), kh.close(), kr.close(), kq.close(), ks.close(), kt.close()
 
 
 def test_reproducible_and_exceptions(capi, ctx, blobs):
