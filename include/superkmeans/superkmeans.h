@@ -744,7 +744,7 @@ class SuperKMeans {
             hip::Check(skm_sync(ctx));
         } else {
             std::vector<float> staged(k * d);
-            for (size_t i = 0; i < k; ++i) std::memcpy(&staged[i * d], data + indices[i] * d, sizeof(float) * d);
+            GatherHostRows(staged.data(), data, indices.data(), k);
             horizontal_centroids.Upload(staged.data(), k * d);
         }
         dbuf<float> rotated(ctx, k * d);
