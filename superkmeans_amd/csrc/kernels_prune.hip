@@ -482,11 +482,11 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
             } else {
                 if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
                 const float4 xv = load_x4<VEC>(xq + V + hb * SKM_H_DIM_SIZE + sub * 4);
-                // 16 survivors per pass: the four gathers of a lane are issued before any of them is used.
-                for (int s0 = 0; s0 < cnt; s0 += 16) {
-                    float4 cv[4];
+                // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.
+                for (int s0 = 0; s0 < cnt; s0 += 32) {
+                    float4 cv[8];
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < 8; ++u) {
                         const int s = s0 + 4 * u + grp;
                         const int cpos = s < cnt ? pos[s] : pos[0];
                         const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
@@ -497,7 +497,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListA
                         }
                     }
 #pragma unroll
-                    for (int u = 0; u < 4; ++u) {
+                    for (int u = 0; u < 8; ++u) {
                         const int s = s0 + 4 * u + grp;
                         float e, part = 0.0f;
                         e = xv.x - cv[u].x; part += e * e;
