@@ -354,7 +354,7 @@ struct PruneListArgs {
 };
 
 template <bool VEC>
-__global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_list_kernel(PruneListArgs a) {
+__global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneListArgs a) {
     __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
     __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
     __shared__ float s_parts[PRUNE_WAVES][16 * 8];  // [block of the group][survivor]
