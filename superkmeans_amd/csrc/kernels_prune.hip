@@ -353,7 +353,7 @@ struct PruneListArgs {
     int n, k, d, vertical_d, partial_d;
 };
 
-template <bool VEC>
+template <bool VEC, bool ACCT>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
 __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneListArgs a) {
     __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
     __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     const int n_hblocks = (d - V) / SKM_H_DIM_SIZE;
     // Accounting counters come in SKM_ACCT_COPIES striped copies (summed by the host) so that the
     // atomics of concurrently running workgroups spread over many addresses.
-    unsigned long long* acct = a.stage_pairs ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
+    unsigned long long* acct = ACCT ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
     const float* xq = a.x + (int64_t) p * d;
     const uint2* list = a.cand + (int64_t) p * a.cap;
     const int sub = lane & 15, grp = lane >> 4;
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
             if (chunk0 + lane < n_cand) entry = list[chunk0 + lane];
         }
         not_pruned_total += (uint32_t) cnt;
-        if (acct && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
+        if (ACCT && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
         if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
         if (cnt == 0) continue;
 
@@ -466,7 +466,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
                 for (; done < G; ++done) {
                     const int entering = __popcll(__ballot(alive));
                     if (entering == 0) break;
-                    if (acct && lane == 0) atomicAdd(&acct[1 + hb + done], (unsigned long long) entering);
+                    if (ACCT && lane == 0) atomicAdd(&acct[1 + hb + done], (unsigned long long) entering);
                     if (alive) my_acc += parts[done * 8 + lane];
                     alive = alive && my_acc < best * a.ratios[dims_seen + (done + 1) * SKM_H_DIM_SIZE];
                 }
@@ -480,7 +480,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
                 hb += G;
                 dims_seen += G * SKM_H_DIM_SIZE;
             } else {
-                if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
+                if (ACCT && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
                 const float4 xv = load_x4<VEC>(xq + V + hb * SKM_H_DIM_SIZE + sub * 4);
                 // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.
                 for (int s0 = 0; s0 < cnt; s0 += 32) {
@@ -517,10 +517,10 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
             // it is (the rule of pdxearch.h:140-143, applied after a step as well as before the first one).  It
             // would otherwise walk all remaining blocks alone, one dependent gather after the other.  With
             // per-step accounting requested it keeps walking, so that the counts are those of the reference.
-            if (cnt == 1 && acct == nullptr && (uint32_t) (base + pos[0]) == prev_top_1) cnt = 0;
+            if (cnt == 1 && !ACCT && (uint32_t) (base + pos[0]) == prev_top_1) cnt = 0;
         }
         if (cnt > 0 && dp < V) {
-            if (acct && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
+            if (ACCT && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
             const int left = V - dp;
             for (int s0 = 0; s0 < cnt; s0 += 4) {
                 const int s = s0 + grp;
@@ -624,10 +624,14 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
     dim3 grid((n_chunk + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
-    if (vec)
-        hipLaunchKernelGGL(prune_list_kernel<true>, grid, block, 0, ctx->stream, a);
+    if (vec && d_stage_pairs)
+        hipLaunchKernelGGL((prune_list_kernel<true, true>), grid, block, 0, ctx->stream, a);
+    else if (vec)
+        hipLaunchKernelGGL((prune_list_kernel<true, false>), grid, block, 0, ctx->stream, a);
+    else if (d_stage_pairs)
+        hipLaunchKernelGGL((prune_list_kernel<false, true>), grid, block, 0, ctx->stream, a);
     else
-        hipLaunchKernelGGL(prune_list_kernel<false>, grid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((prune_list_kernel<false, false>), grid, block, 0, ctx->stream, a);
     return check_hip(hipGetLastError(), "prune_list_kernel launch");
 }
 
