@@ -254,7 +254,9 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
     }
 
     static constexpr size_t FINE_HELPERS_DEFAULT = 8;  // concurrent fine-phase problems when n_threads is 0
-    static constexpr size_t FINE_HELPERS_MAX = 16;
+    // Every helper thread waits for its stream by polling; sixteen of them on a sixteen-core share of the host were
+    // throttled and took four times as long as twelve.
+    static constexpr size_t FINE_HELPERS_MAX = 12;
 
     // What every fine-phase problem reads (device pointers of the owner, host tables) and where it writes.
     struct FineInputs {
