@@ -31,7 +31,10 @@ def test_pdxify_rejects_bad_split(capi, ctx):
                                             (70000, 64, 70000, 8), (257, 1536, 1, 2),
                                             # few centroids, long segments: columns of a centroid spread over several
                                             # workgroups, 32 rows in flight per thread; the order of additions is the same
-                                            (40000, 1024, 9, 4), (50000, 512, 20, 2)])
+                                            (40000, 1024, 9, 4), (50000, 512, 20, 2),
+                                            # ragged column groups of the row-sum kernel: 33 and 5 float4 lanes, 20 and 200
+                                            # single-float lanes (the last wavefront of a centroid is partly idle)
+                                            (30000, 132, 3000, 2), (20000, 20, 3000, 1), (5000, 20, 10, 1), (30000, 200, 600, 3)])
 def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
     g = np.random.default_rng(n + d)
     X = g.standard_normal((n, d)).astype(np.float32)

@@ -14,10 +14,11 @@ def _rel_l2(a, b):
 
 
 def test_host_tables_identical_to_oracle(capi, ctx, oracle):
-    """Same seed -> same rotation matrix and ratios in both implementations (bit for bit).  From d = 192 on the
+    """Same seed -> same rotation matrix and ratios in both implementations (bit for bit).  From d = 384 on the
     library factorises on the device (skm_householder_q) with the host routine's operation order; the oracle
-    factorises on the CPU: 256, 300 (ragged last column block) and 1024 compare the two."""
-    for d in (64, 100, 256, 300, 1024):
+    factorises on the CPU: 384 and up compare the two (1024 with 16 columns per workgroup, 1300 with 8 and a ragged
+    last group)."""
+    for d in (64, 100, 256, 390, 1024, 1300):
         m, r = capi.pruner_tables(d, 1.5, 42)
         assert np.array_equal(m, oracle.rotation_matrix(d, 42))
         assert np.array_equal(r, oracle.ratios(d, 1.5))
