@@ -181,3 +181,22 @@ def test_bad_arguments_are_rejected(capi, ctx):
     with pytest.raises(capi.SkmError):
         capi.check(ctx.lib.skm_rotate(ctx.handle, x.ptr, 4, 8, x.ptr, x.ptr))  # in place
     x.free()
+
+
+def test_upload_on_the_transfer_stream_orders_before_later_work(capi, ctx):
+    """skm_upload_overlapped copies on the context's second stream; what is queued afterwards must see the data, what
+    was queued before keeps running.  Slabs are uploaded one after the other, each followed by the norms of its rows."""
+    g = np.random.default_rng(5)
+    n, d, slab = 60000, 512, 7000
+    X = g.standard_normal((n, d)).astype(np.float32)
+    dX, out = ctx.empty((n, d)), ctx.empty(n)
+    for r0 in range(0, n, slab):
+        m = min(slab, n - r0)
+        rows = np.ascontiguousarray(X[r0:r0 + m])
+        capi.check(ctx.lib.skm_upload_overlapped(ctx.handle, dX.ptr + r0 * d * 4, rows.ctypes.data, m * d * 4))
+        capi.check(ctx.lib.skm_norms(ctx.handle, dX.ptr + r0 * d * 4, m, d, d, out.ptr + r0 * 4))
+    ctx.sync()
+    assert np.array_equal(dX.download(), X)
+    assert np.allclose(out.download(), (X.astype(np.float64) ** 2).sum(1), rtol=1e-5)
+    dX.free(), out.free()
+
