@@ -26,6 +26,23 @@ def test_host_tables_identical_to_oracle(capi, ctx, oracle):
     assert not np.array_equal(m2, capi.pruner_tables(64, 1.5, 42)[0])  # test_rotation.cpp:337-387
 
 
+def test_device_factorisation_rejects_what_it_cannot_hold(capi, ctx):
+    """skm_householder_q keeps all rows of eight columns in LDS: beyond d = 2272 it reports an error (the pruner then
+    factorises on the host) instead of launching."""
+    d = 2400
+    a = np.zeros((d, d), dtype=np.float64)
+    out = np.zeros((d, d), dtype=np.float32)
+    with pytest.raises(capi.SkmError, match="out of range"):
+        capi.check(ctx.lib.skm_householder_q(ctx.handle, a.ctypes.data, d, out.ctypes.data))
+    with pytest.raises(capi.SkmError, match="null"):
+        capi.check(ctx.lib.skm_householder_q(ctx.handle, None, 64, out.ctypes.data))
+    # the identity factorises to a signed identity: every reflector only flips its diagonal entry
+    d = 400
+    q = np.zeros((d, d), dtype=np.float32)
+    capi.check(ctx.lib.skm_householder_q(ctx.handle, np.eye(d).ctypes.data, d, q.ctypes.data))
+    assert np.array_equal(np.abs(q), np.eye(d, dtype=np.float32))
+
+
 def _pruned_iteration_on_gpu(capi, ctx, oracle, Xrot, C, prev, partial_d, ratios):
     """One pruned iteration (search + update + scaling) through the stage-level C ABI."""
     import ctypes
