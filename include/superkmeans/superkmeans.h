@@ -197,15 +197,19 @@ class SuperKMeans {
         return std::max<size_t>(256, rows / 256 * 256);
     }
 
-    /** Assign on device-resident inputs; writes n_vectors indices to d_out_assignments (asynchronous). */
+    /** Assign on device-resident inputs; writes n_vectors indices to d_out_assignments.  Queued on the object's
+     *  context, not waited for: read the output after skm_sync (or through a download on the same context). */
     void AssignDevice(const vector_value_t* d_vectors, const vector_value_t* d_centroids, const size_t n_vectors,
                       const size_t n_centroids, uint32_t* d_out_assignments) {
-        dbuf<float> v_norms(ctx, n_vectors), c_norms(ctx, n_centroids), dist(ctx, n_vectors);
-        hip::Check(skm_norms(ctx, d_vectors, n_vectors, d, d, v_norms.get()));
-        hip::Check(skm_norms(ctx, d_centroids, n_centroids, d, d, c_norms.get()));
-        hip::Check(skm_assign_full(ctx, d_vectors, n_vectors, d_centroids, n_centroids, d, v_norms.get(),
-                                   c_norms.get(), d_out_assignments, dist.get()));
-        hip::Check(skm_sync(ctx));  // the scratch buffers above are released on return
+        // norms and distances live in buffers that the object keeps between calls (allocating and releasing
+        // them costs a third of a millisecond per call, and a release waits for the device)
+        if (assign_v_norms.size() < n_vectors) assign_v_norms.Reset(ctx, n_vectors);
+        if (assign_dist.size() < n_vectors) assign_dist.Reset(ctx, n_vectors);
+        if (assign_c_norms.size() < n_centroids) assign_c_norms.Reset(ctx, n_centroids);
+        hip::Check(skm_norms(ctx, d_vectors, n_vectors, d, d, assign_v_norms.get()));
+        hip::Check(skm_norms(ctx, d_centroids, n_centroids, d, d, assign_c_norms.get()));
+        hip::Check(skm_assign_full(ctx, d_vectors, n_vectors, d_centroids, n_centroids, d, assign_v_norms.get(),
+                                   assign_c_norms.get(), d_out_assignments, assign_dist.get()));
     }
 
     /** Pruned assignment of the training points, seeded with the assignments found by Train. */
@@ -961,7 +965,8 @@ class SuperKMeans {
     skm_ctx* ctx = nullptr;
     std::shared_ptr<pruner_t> pruner;
 
-    // Device state (names follow the reference's members, superkmeans.h:1470-1480)
+    // Device state (names follow the reference's members, superkmeans.h:1470-1480).  Declared after `context`:
+    // members are destroyed in reverse order and a buffer releases its memory through the context.
     dbuf<float> centroids;                     // PDX layout
     dbuf<float> horizontal_centroids;          // row-major: raw init rows -> sums -> means
     dbuf<float> prev_centroids;                // centroids the current iteration searches against
@@ -972,6 +977,7 @@ class SuperKMeans {
     dbuf<float> data_norms;
     dbuf<float> centroid_norms;
     dbuf<float> training_data;  // rotated samples (unused when the caller's device buffer is used in place)
+    dbuf<float> assign_v_norms, assign_c_norms, assign_dist;  // scratch of AssignDevice, kept between calls
 
     // Host state
     std::unique_ptr<uint32_t[]> cluster_sizes;

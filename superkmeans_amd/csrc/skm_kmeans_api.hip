@@ -171,7 +171,10 @@ int skm_kmeans_assign_device(skm_kmeans* km, const float* d_vectors, const float
                              size_t n_centroids, uint32_t* d_out_assignments) {
     if (!km || !d_vectors || !d_centroids || !d_out_assignments)
         return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_assign_device: null argument");
-    SKM_API_GUARD(km->base()->AssignDevice(d_vectors, d_centroids, n_vectors, n_centroids, d_out_assignments));
+    SKM_API_GUARD({
+        km->base()->AssignDevice(d_vectors, d_centroids, n_vectors, n_centroids, d_out_assignments);
+        skmeans::hip::Check(skm_sync(km->base()->GetContext()));
+    });
 }
 
 int skm_kmeans_assign_training_points(skm_kmeans* km, const float* h_vectors, const float* h_centroids,
