@@ -51,6 +51,8 @@ struct GemmShape {
 };
 using GemmSmall = GemmShape<2, 2, 2, 2, 2>;
 using GemmBig = GemmShape<2, 4, 4, 2, 1>;
+// 128 x 64: for problems of a few hundred 128 x 128 tiles, where whole tiles leave part of the chip idle in the last round.
+using GemmHalf = GemmShape<2, 2, 2, 1, 2>;
 // (32 FM) x 128: a few M rows against all N rows, bound by the loads of the N operand.  Used for the centroids left
 // over when k is up to 128 rows more than a multiple of the large shape's 256.
 template <int FM>

@@ -99,6 +99,22 @@ def test_assign_full_workgroup_tile_shape_never_changes_a_bit(capi, ctx, oracle,
     assert np.allclose(gd[-m:], bbest, rtol=1e-4, atol=1e-5)
 
 
+def test_assign_full_half_width_tiles_never_change_a_bit(capi, ctx, oracle):
+    """39,000 points x 256 centroids are 610 tiles of 128 x 128 on 512 workgroup slots: the search then uses tiles of
+    128 x 64; slices of 19,500 points (314 tiles) use whole tiles.  Same accumulation order, same bits."""
+    g = np.random.default_rng(39)
+    n, k, d = 39000, 256, 70
+    X = g.standard_normal((n, d)).astype(np.float32)
+    C = g.standard_normal((k, d)).astype(np.float32)
+    gi, gd, _ = _assign_full(capi, ctx, X, C)
+    for i0 in (0, 19500):
+        si, sd, _ = _assign_full(capi, ctx, X[i0:i0 + 19500], C)
+        assert np.array_equal(gi[i0:i0 + 19500], si) and np.array_equal(gd[i0:i0 + 19500], sd)
+    bi, bbest, bsecond = oracle.brute_force(X[-3000:], C)
+    tie = (bsecond - bbest) <= 1e-4 * np.maximum(bbest, 1e-12)
+    assert np.all((gi[-3000:] == bi) | tie)
+
+
 def test_rotate_large_tile_shape_equals_small_tile_shape(capi, ctx, oracle):
     n, d = 270000, 256  # 1,055 tiles of 256 x 256
     Q = oracle.rotation_matrix(d, seed=7)
