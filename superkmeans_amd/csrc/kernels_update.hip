@@ -72,13 +72,6 @@ __global__ __launch_bounds__(256) void segment_bounds_kernel(
     for (uint32_t c = first; c <= key; ++c) offsets[c] = (uint32_t) i;
 }
 
-__global__ __launch_bounds__(256) void sizes_from_offsets_kernel(
-    const uint32_t* __restrict__ offsets, uint32_t k, uint32_t* __restrict__ sizes
-) {
-    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c < k) sizes[c] = offsets[c + 1] - offsets[c];
-}
-
 // Pass 1 of a radix step: digit histogram of one tile, stored digit-major so that one exclusive
 // scan over [digit][tile] yields the global base of every (digit, tile) pair.
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
@@ -153,10 +146,11 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
 // workgroup per centroid, one column per thread, rows in ascending point id.
 __global__ __launch_bounds__(256) void segment_sum_columns_kernel(
     const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
-    const uint32_t* __restrict__ offsets, float* __restrict__ sums
+    const uint32_t* __restrict__ offsets, float* __restrict__ sums, uint32_t* __restrict__ sizes
 ) {
     const uint32_t c = blockIdx.x;
     const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
+    if (threadIdx.x == 0) sizes[c] = j1 - j0;
     float* out = sums + (size_t) c * d;
     for (size_t t = threadIdx.x; t < d; t += blockDim.x) {
         float acc = 0.0f;
@@ -175,12 +169,13 @@ __global__ __launch_bounds__(256) void segment_sum_columns_kernel(
 template <int W, int ROWS>
 __global__ __launch_bounds__(64) void segment_sum_deep_kernel(
     const float* __restrict__ x, size_t d, const uint32_t* __restrict__ sorted_ids,
-    const uint32_t* __restrict__ offsets, float* __restrict__ sums, uint32_t groups
+    const uint32_t* __restrict__ offsets, float* __restrict__ sums, uint32_t* __restrict__ sizes, uint32_t groups
 ) {
     static_assert(ROWS <= 64, "lane u prepares the address of row u of a batch");
     typedef float vec_t __attribute__((ext_vector_type(W)));
     const uint32_t c = blockIdx.x / groups, g = blockIdx.x % groups;
     const uint32_t j0 = offsets[c], j1 = offsets[c + 1];
+    if (g == 0 && threadIdx.x == 0) sizes[c] = j1 - j0;  // the cluster's size is the length of its segment
     const size_t t = (size_t) g * 64 + threadIdx.x;  // column group of this lane
     const size_t n_groups = d / W;
     const size_t t_load = t < n_groups ? t : n_groups - 1;  // lanes past the last column load it again and store nothing
@@ -413,9 +408,6 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         sorted_ids = vals_a;
         SKM_TRY(skm_fill_u32(ctx, offsets, 0u, k + 1));
     }
-    hipLaunchKernelGGL(sizes_from_offsets_kernel, dim3((unsigned) ((k + 255) / 256)), dim3(256), 0, ctx->stream, offsets,
-                       (uint32_t) k, d_out_sizes);
-    SKM_HIP_TRY(hipGetLastError());
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
     if (vec) {
@@ -426,13 +418,13 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         SKM_REQUIRE(k * groups <= 0x7fffffffULL, "k * d too large for one launch");
         dim3 grid((unsigned) (k * groups));
         if (w == 4)
-            hipLaunchKernelGGL((segment_sum_deep_kernel<4, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+            hipLaunchKernelGGL((segment_sum_deep_kernel<4, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, d_out_sizes, (uint32_t) groups);
         else if (w == 2)
-            hipLaunchKernelGGL((segment_sum_deep_kernel<2, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+            hipLaunchKernelGGL((segment_sum_deep_kernel<2, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, d_out_sizes, (uint32_t) groups);
         else
-            hipLaunchKernelGGL((segment_sum_deep_kernel<1, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, (uint32_t) groups);
+            hipLaunchKernelGGL((segment_sum_deep_kernel<1, 32>), grid, dim3(64), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, d_out_sizes, (uint32_t) groups);
     } else {
-        hipLaunchKernelGGL(segment_sum_columns_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums);
+        hipLaunchKernelGGL(segment_sum_columns_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, d_out_sizes);
     }
     return check_hip(hipGetLastError(), "segment sum launch");
 }
