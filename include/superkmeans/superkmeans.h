@@ -147,6 +147,11 @@ class SuperKMeans {
         context = std::make_shared<hip::Context>(0);
         ctx = context->get();
         pruner = std::move(shared_pruner);
+        // same rule as the public constructor (reference superkmeans.h:137-139): centroids of data that was
+        // never rotated here must not be "un-rotated"
+        if (this->config.data_already_rotated) {
+            this->config.unrotate_centroids = false;
+        }
     }
 
   public:
