@@ -110,6 +110,20 @@ int skm_pdxify(skm_ctx* ctx, const float* d_c, size_t k, size_t d, size_t vertic
 int skm_assign_full(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, size_t k, size_t d,
                     const float* d_xnorm, const float* d_cnorm, uint32_t* d_out_idx, float* d_out_dist);
 
+/* skm_assign_full for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical results; the per-(granule of centroids, point) minima that skm_assign_full keeps in the context's
+ * workspace live in a static device array of SKM_NOALLOC_SCRATCH_BYTES that every GPU running the library holds
+ * until the process ends.  The call allocates and releases nothing (its address was resolved by skm_ctx_create)
+ * and records no device timers.  Points are processed in chunks that fit the array, so n is not limited;
+ * k > SKM_NOALLOC_MAX_CENTROIDS is rejected with SKM_ERR_INVALID.  All calls on one GPU share the array: calls
+ * that overlap in time on the same GPU (two contexts, two threads) race; nothing in it has to be cleared
+ * between calls (every entry a merge reads was written by the launch before it). */
+#define SKM_NOALLOC_SCRATCH_BYTES (32u << 20)
+#define SKM_NOALLOC_MAX_CENTROIDS 2097152 /* 128 points x ceil(k / 64) granules x 8 bytes fill the array */
+int skm_assign_full_noalloc(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, size_t k, size_t d,
+                            const float* d_xnorm, const float* d_cnorm, uint32_t* d_out_idx, float* d_out_dist);
+
 /* BatchComputer::FindNearestNeighborWithPruning (batch_computers.h:297-409) with
  * PDXearch::Top1PartialSearchWithThresholdAndPartialDistances / Prune / SetBestCandidate
  * (pdx/pdxearch.h:118-238,266-327).

@@ -44,6 +44,7 @@ _PROTOTYPES = {
     "skm_transpose": (c_int, [c_void_p, _F, c_size_t, c_size_t, _F]),
     "skm_pdxify": (c_int, [c_void_p, _F, c_size_t, c_size_t, c_size_t, _F, _F]),
     "skm_assign_full": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_size_t, _F, _F, _F, _F]),
+    "skm_assign_full_noalloc": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_size_t, _F, _F, _F, _F]),
     "skm_assign_pruned": (
         c_int,
         [c_void_p, _F, c_size_t, _F, _F, _F, c_size_t, c_size_t, c_size_t, c_uint32, _F, _F, _F, _F, _F,

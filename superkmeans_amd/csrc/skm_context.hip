@@ -144,8 +144,11 @@ int skm_ctx_create(int device, skm_ctx** out_ctx) {
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(SKM_ERR_NO_DEVICE, "skm_ctx_create: device %d is %s; this library is built for gfx950 only",
                          device, prop.gcnArchName);
+    void* noalloc_scratch = nullptr;
+    SKM_TRY(resolve_noalloc_scratch(device, &noalloc_scratch));
     skm_ctx* ctx = new skm_ctx();
     ctx->device = device;
+    ctx->noalloc_scratch = noalloc_scratch;
     hipError_t e = hipStreamCreate(&ctx->stream);
     if (e != hipSuccess) {
         delete ctx;

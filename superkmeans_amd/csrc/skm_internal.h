@@ -34,6 +34,8 @@ struct skm_ctx {
     // Small pinned host buffer for scalar results.
     void* h_pinned = nullptr;
     size_t h_pinned_bytes = 0;
+    // Address, on this context's device, of the library's static scratch array (skm_assign_full_noalloc).
+    void* noalloc_scratch = nullptr;
     bool prof = false;
     std::map<std::string, skm_scope_timer> timers;
     std::vector<skm_pending_interval> pending;
@@ -79,6 +81,10 @@ class ScopedStage {
 };
 
 int resolve_pending(skm_ctx* ctx);
+
+// Device address of the static scratch array of skm_assign_full_noalloc on `device` (which must be the current
+// device); resolved once per device and kept.
+int resolve_noalloc_scratch(int device, void** out);
 
 // ---- launchers implemented in the kernel translation units ----
 

@@ -2,8 +2,30 @@
 #include "skm_internal.h"
 
 #include <algorithm>
+#include <mutex>
+
+// Scratch of skm_assign_full_noalloc: per-(granule, point) minima of one chunk of points.  One copy per device
+// that loads the library, held until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; kernels and copies get the resolved device address.
+static __device__ __align__(256) unsigned char scratch[SKM_NOALLOC_SCRATCH_BYTES];
 
 namespace skm {
+
+int resolve_noalloc_scratch(int device, void** out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex lock;
+    static void* resolved[MAX_DEVICES] = {};
+    if (device < 0 || device >= MAX_DEVICES) return set_error(SKM_ERR_INVALID, "device index out of range");
+    std::lock_guard<std::mutex> guard(lock);
+    if (!resolved[device]) {
+        void* ptr = nullptr;
+        SKM_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return set_error(SKM_ERR_HIP, "hipGetSymbolAddress returned a null address");
+        resolved[device] = ptr;
+    }
+    *out = resolved[device];
+    return SKM_OK;
+}
 
 // One wavefront per row; lane-strided accumulation then a fixed butterfly, so the result does not
 // depend on launch geometry.
@@ -138,6 +160,34 @@ int skm_assign_full(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, 
             SKM_TRY(launch_merge_granules(ctx, (const uint2*) scratch, (int) m, (int) k, granule, d_out_idx + i0,
                                           d_out_dist + i0));
         }
+    }
+    return SKM_OK;
+}
+
+int skm_assign_full_noalloc(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, size_t k, size_t d,
+                            const float* d_xnorm, const float* d_cnorm, uint32_t* d_out_idx, float* d_out_dist) {
+    SKM_REQUIRE(ctx, "null context");
+    if (n == 0) return SKM_OK;
+    SKM_REQUIRE(d_x && d_c && d_xnorm && d_cnorm && d_out_idx && d_out_dist, "null pointer");
+    SKM_REQUIRE(k > 0 && d > 0, "k and d must be positive");
+    SKM_REQUIRE(d <= (1u << 20), "d out of range");
+    if (k > SKM_NOALLOC_MAX_CENTROIDS)
+        return set_error(SKM_ERR_INVALID, "skm_assign_full_noalloc: k = %zu exceeds the limit of %d centroids that the "
+                         "static scratch of %d MiB allows; use skm_assign_full", k, SKM_NOALLOC_MAX_CENTROIDS,
+                         (int) (SKM_NOALLOC_SCRATCH_BYTES >> 20));
+    SKM_REQUIRE(ctx->noalloc_scratch, "static scratch was not resolved for this context");
+    // Same two kernels as skm_assign_full; the granule minima of a chunk of points live in the static array.
+    // No device timers here: they take events from a pool that may have to create them.
+    const size_t n_granules = (k + 63) / 64;  // the smallest granule: an upper bound for every chunk
+    size_t chunk = SKM_NOALLOC_SCRATCH_BYTES / (n_granules * sizeof(uint2));
+    chunk = (chunk / 128) * 128;  // >= 128 by the limit on k
+    uint2* granule_min = (uint2*) ctx->noalloc_scratch;
+    for (size_t i0 = 0; i0 < n; i0 += chunk) {
+        const size_t m = std::min(chunk, n - i0);
+        const int granule = gemm_argmin_granule((int) k, (int) m);
+        SKM_TRY(launch_gemm_argmin(ctx, d_c, (int) k, d_x + i0 * d, (int) m, (int) d, (int64_t) d, (int64_t) d,
+                                   d_xnorm + i0, d_cnorm, granule_min, granule));
+        SKM_TRY(launch_merge_granules(ctx, granule_min, (int) m, (int) k, granule, d_out_idx + i0, d_out_dist + i0));
     }
     return SKM_OK;
 }
