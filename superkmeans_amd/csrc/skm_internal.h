@@ -115,6 +115,11 @@ int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const f
 int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                            const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
                            uint2* cand, uint32_t cap);
+// The same for short d' (the points stay in registers); `serves` says whether a call qualifies.
+bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, int n, int partial_d, int64_t ld);
+int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
+                                      const float* xnorm_p, const float* cnorm_p, const float* thr0,
+                                      uint32_t* cand_count, uint2* cand, uint32_t cap);
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
                          const float* ratios, int partial_d, float* best0, float* thr0);
 int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,

@@ -12,6 +12,8 @@
 #include "skm_internal.h"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstdio>
 #include <vector>
 
 namespace skm {
@@ -111,8 +113,19 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         }
         {
             ScopedStage st(ctx, "search/blas");
-            SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
-                                           d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
+            if (gemm_candidates_stationary_serves(d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d) &&
+                !getenv("SKM_CAND_OLD"))
+                SKM_TRY(launch_gemm_candidates_stationary(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d,
+                                                          d_xnorm_p + i0, d_cnorm_p, d_thr0, d_cand_count,
+                                                          (uint2*) ws_cand, cap));
+            else
+                SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
+                                               d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
+        }
+        if (getenv("SKM_CS_DBG") && (atoi(getenv("SKM_CS_DBG")) & 16)) {
+            double tot = 0;
+            SKM_TRY(reduce_u32_sum_to_host(ctx, d_cand_count, m, &tot));
+            fprintf(stderr, "[dbg] d'=%u candidates emitted: %.0f = %.4f %% of pairs\n", partial_d, tot, 100.0 * tot / ((double) m * k));
         }
         SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over));
         {
