@@ -55,6 +55,12 @@ int skm_sync(skm_ctx* ctx);
  * 288 GB of HBM: large enough that the headline shapes run as one launch per stage). */
 int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
 
+/* Which kernel computes the partial distances of skm_assign_pruned (tuning and test knob; results do not depend on
+ * it): 0 = automatic (default: the register-stationary kernel for partial_d <= 160 and at least 131,072 points per
+ * call, the tiled 128 x 128 kernel otherwise), 1 = always the tiled kernel, 2 = the register-stationary kernel
+ * whenever partial_d <= 160 and the rows are 16-byte aligned, whatever the number of points. */
+int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which);
+
 /* Device memory and transfers (stand in for the reference's std::unique_ptr<float[]> buffers,
  * superkmeans.h:191-201). */
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr);

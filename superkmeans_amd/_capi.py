@@ -26,6 +26,7 @@ _PROTOTYPES = {
     "skm_ctx_destroy": (c_int, [c_void_p]),
     "skm_sync": (c_int, [c_void_p]),
     "skm_ctx_set_workspace_limit": (c_int, [c_void_p, c_size_t]),
+    "skm_ctx_set_candidate_kernel": (c_int, [c_void_p, c_int]),
     "skm_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "skm_free": (c_int, [c_void_p, c_void_p]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),

@@ -37,13 +37,9 @@
 #include "gemm_core.h"
 #include "skm_internal.h"
 
-#include <cstdio>
-#include <cstdlib>
-
 namespace skm {
 
-constexpr int CS_THREADS = 256;
-constexpr int CS_POINTS = 256;  // per workgroup
+constexpr int CS_POINTS = 256;  // per workgroup: 4 wavefronts of 64 points (d' <= 88) or 8 wavefronts of 32 points
 constexpr int CS_TN = 64;       // centroids per tile
 constexpr float CS_SLACK = 1.0f / 131072.0f;
 constexpr float CS_NEVER = -1.5e38f;  // addend of rows and columns that must not pass
@@ -62,57 +58,60 @@ __device__ __forceinline__ int cs_row_of_bit(int bit) {
     return 8 * ((bit & 15) >> 2) + 4 * (bit >> 4) + (bit & 3);
 }
 
-template <int NG>  // groups of 8 columns: ceil(d' / 8)
-__global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kernel(
+// NG: groups of 8 columns, ceil(d' / 8).  FM: 32-point accumulator block rows per wavefront (2 or 1); the wavefronts of
+// a workgroup are 8 / FM, so that it always owns 256 points and streams a centroid tile once for all of them.
+template <int NG, int FM>
+__global__ __launch_bounds__(512 / FM, FM) void gemm_candidates_stationary_kernel(
     const float* __restrict__ C, int M, const float* __restrict__ X, int N, int K, int64_t ld,
     const float* __restrict__ xnorm, const float* __restrict__ cnorm, const float* __restrict__ thr0,
-    uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap, int dbg
+    uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap
 ) {
+    constexpr int WAVES = 8 / FM, CS_THREADS = 64 * WAVES;
     constexpr int S = NG * 8 + 4;           // LDS row stride in floats: 16-byte fragment reads of 32 rows hit all banks
     constexpr int CHUNKS = CS_TN * NG * 2;  // 16-byte pieces of a tile
     constexpr int NL = (CHUNKS + CS_THREADS - 1) / CS_THREADS;
     constexpr bool RAGGED = CHUNKS % CS_THREADS != 0;  // NG odd: the last load of half the threads has no piece
     extern __shared__ __attribute__((aligned(16))) float cs_lds[];
     float (*Bs)[CS_TN * S] = reinterpret_cast<float (*)[CS_TN * S]>(cs_lds);  // [2]: centroid tiles
-    float* const dump_all = cs_lds + 2 * CS_TN * S;                           // [4][32 bits][64 centroids]
-    CsPoint* const table_all = reinterpret_cast<CsPoint*>(dump_all + 4 * 32 * 64);  // [4][2 block rows][32 bits]
+    float* const dump_all = cs_lds + 2 * CS_TN * S;                                     // [WAVES][32 bits][64 centroids]
+    CsPoint* const table_all = reinterpret_cast<CsPoint*>(dump_all + WAVES * 32 * 64);  // [WAVES][FM block rows][32 bits]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5;  // which 4 of every 8 accumulator rows / which 4 of every 8 columns this lane feeds
-    const int wave_pt0 = blockIdx.x * CS_POINTS + wave * 64;
+    const int wave_pt0 = blockIdx.x * CS_POINTS + wave * (32 * FM);
     float* const dump = dump_all + wave * (32 * 64);
-    CsPoint* const table = table_all + wave * 64;
+    CsPoint* const table = table_all + wave * (32 * FM);
 
     // ---- per point: table entry (lane j fills entry j = 32 mb + bit) and row addend of the sign test ----
-    {
+    if (lane < 32 * FM) {
         const int local = (lane & 32) + cs_row_of_bit(lane & 31);
         const int pt = wave_pt0 + local;
         CsPoint e;
         e.xn = pt < N ? xnorm[pt] : 0.0f;
-        e.thr = (pt < N && !(dbg & 2)) ? thr0[pt] : -3.0e38f;
+        e.thr = pt < N ? thr0[pt] : -3.0e38f;
         e.list_off = (uint32_t) local * cap * (uint32_t) sizeof(uint2);
         e.count = 0u;
         table[lane] = e;
     }
     // MFMA row operand of the extra step: k = 0 (lanes 0-31) supplies (thr - |x|^2) / 2 plus slack for point
     // mb * 32 + lane, k = 1 (lanes 32-63) multiplies the column addend by 1
-    float a_aug[2];
+    float a_aug[FM];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
+    for (int mb = 0; mb < FM; ++mb) {
         const int pt = wave_pt0 + mb * 32 + (lane & 31);
         const float xn = pt < N ? xnorm[pt] : 0.0f;
-        const float thr = (pt < N && !(dbg & 2)) ? thr0[pt] : -3.0e38f;
+        const float thr = pt < N ? thr0[pt] : -3.0e38f;
         a_aug[mb] = half ? 1.0f : 0.5f * (thr - xn) + CS_SLACK * (xn + fabsf(thr));
     }
     // first list of the wavefront; a point's list starts list_off bytes further
     char* const wave_lists = reinterpret_cast<char*>(cand + (int64_t) wave_pt0 * cap);
 
     // ---- point fragments: a[kg][mb] = columns kg * 8 + half * 4 .. + 3 of point mb * 32 + lane % 32 ----
-    floatx4 a[NG][2];
+    floatx4 a[NG][FM];
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
+    for (int mb = 0; mb < FM; ++mb) {
         int q = wave_pt0 + mb * 32 + (lane & 31);
         q = q < N ? q : N - 1;
         const float* row = X + (int64_t) q * ld + half * 4;
@@ -173,9 +172,9 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
     };
 
     // acc.v[mb][nb][r] of lane l: point mb * 32 + 8 (r / 4) + 4 (l / 32) + r % 4, centroid nb * 32 + l % 32
-    WaveAcc acc;
+    WaveAccT<FM, 2> acc;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < FM; ++mb)
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
@@ -198,17 +197,16 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                if (kg == 0 && i == 0) {
-                    const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][0][i], fb0[i], zero, 0, 0, 0);
-                    acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][0][i], fb1[i], zero, 0, 0, 0);
-                    acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][1][i], fb0[i], zero, 0, 0, 0);
-                    acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][1][i], fb1[i], zero, 0, 0, 0);
-                } else {
-                    acc.v[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][0][i], fb0[i], acc.v[0][0], 0, 0, 0);
-                    acc.v[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][0][i], fb1[i], acc.v[0][1], 0, 0, 0);
-                    acc.v[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][1][i], fb0[i], acc.v[1][0], 0, 0, 0);
-                    acc.v[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][1][i], fb1[i], acc.v[1][1], 0, 0, 0);
+#pragma unroll
+                for (int mb = 0; mb < FM; ++mb) {
+                    if (kg == 0 && i == 0) {
+                        const floatx16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                        acc.v[mb][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][mb][i], fb0[i], zero, 0, 0, 0);
+                        acc.v[mb][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][mb][i], fb1[i], zero, 0, 0, 0);
+                    } else {
+                        acc.v[mb][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][mb][i], fb0[i], acc.v[mb][0], 0, 0, 0);
+                        acc.v[mb][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kg][mb][i], fb1[i], acc.v[mb][1], 0, 0, 0);
+                    }
                 }
             }
             if (kg + 1 < NG) {
@@ -227,15 +225,22 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
         b_aug[1] = half ? (own_live ? -0.5f * (1.0f - CS_SLACK) * cn_own : CS_NEVER) : 1.0f;
         const uint32_t centroid = (uint32_t) (tile * CS_TN + lane);
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < FM; ++mb) {
+            // dump[bit][centroid] = product of the point of that bit with that centroid.  Written for every block
+            // row, candidates or not: LDS traffic runs beside the MFMAs, vector instructions do not, and with the
+            // products safe in LDS the sign test may overwrite the accumulators (a copy would cost 32 moves).
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dump[(half * 16 + r) * 64 + nb * 32 + (lane & 31)] = acc.v[mb][nb][r];
             uint32_t negative[2];
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
-                const floatx16 t = __builtin_amdgcn_mfma_f32_32x32x2f32(a_aug[mb], b_aug[nb], acc.v[mb][nb], 0, 0, 0);
+                acc.v[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_aug[mb], b_aug[nb], acc.v[mb][nb], 0, 0, 0);
                 uint32_t bits = 0;
 #pragma unroll
-                for (int r = 15; r >= 0; --r) bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(t[r]), 31);
-                negative[nb] = bits;  // bit r: t[r] carries a set sign bit (no candidate)
+                for (int r = 15; r >= 0; --r) bits = __builtin_amdgcn_alignbit(bits, __float_as_uint(acc.v[mb][nb][r]), 31);
+                negative[nb] = bits;  // bit r: the value carries a set sign bit (no candidate)
             }
             // lanes 0-31 keep their low-row bits of column block 0 and receive its high-row bits from lanes 32-63;
             // lanes 32-63 receive the low-row bits of column block 1 from lanes 0-31 and keep their high-row bits:
@@ -243,13 +248,7 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
             const auto sw = __builtin_amdgcn_permlane32_swap(negative[0], negative[1], false, false);
             uint32_t mask = ~((sw[0] & 0xffffu) | (sw[1] << 16));
             if (__builtin_amdgcn_ballot_w64(mask != 0u) == 0ull) continue;
-            // dump[bit][centroid] = product of the point of that bit with that centroid
-#pragma unroll
-            for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) dump[(half * 16 + r) * 64 + nb * 32 + (lane & 31)] = acc.v[mb][nb][r];
             __builtin_amdgcn_wave_barrier();  // LDS serves a wavefront's requests in order: the reads below see the writes
-            if (dbg & 4) continue;
             CsPoint* const points = table + mb * 32;
             for (;;) {
                 const bool active = mask != 0u;
@@ -286,7 +285,7 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
     fetch(0, 0, fb0, fb1);
     for (int t = 0; t <= tiles; ++t) {
         publish((t + 1) & 1);
-        if (!(dbg & 1)) emit(t - 1);
+        emit(t - 1);
         request(t + 2);
         request_norms(t);
         __builtin_amdgcn_sched_barrier(0);
@@ -295,36 +294,39 @@ __global__ __launch_bounds__(CS_THREADS, 2) void gemm_candidates_stationary_kern
         __syncthreads();  // every read of buffer t & 1 has returned, tile t + 1 is complete in the other one
         fetch((t + 1) & 1, 0, fb0, fb1);
     }
-    {
+    if (lane < 32 * FM) {
         const int pt = wave_pt0 + (lane & 32) + cs_row_of_bit(lane & 31);
         if (pt < N) cand_count[pt] = table[lane].count;
     }
 }
 
-// The largest number of 8-column groups whose point fragments fit the register file next to the accumulators
-// (2 wavefronts per SIMD, 256 registers each) and whose two centroid tiles fit LDS twice over next to the
-// wavefronts' scratch.
-constexpr int CS_MAX_GROUPS = 11;
+// Up to 11 groups of 8 columns a wavefront holds the fragments of 64 points next to its 64 x 64 accumulators
+// (2 wavefronts per SIMD, 256 registers each) and two workgroups of 4 wavefronts share a CU; from 12 to 20 groups
+// it holds 32 points, and one workgroup of 8 wavefronts has the CU's LDS to itself.
+constexpr int CS_MAX_GROUPS_WIDE = 11;
+constexpr int CS_MAX_GROUPS = 20;
 
 template <int NG>
 static int launch_stationary(skm_ctx* ctx, dim3 grid, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                              const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
                              uint2* cand, uint32_t cap) {
-    const size_t lds_bytes = (2 * CS_TN * (NG * 8 + 4) + 4 * 32 * 64) * sizeof(float) + 4 * 64 * sizeof(CsPoint);
+    constexpr int FM = NG <= CS_MAX_GROUPS_WIDE ? 2 : 1;
+    constexpr int WAVES = 8 / FM;
+    const size_t lds_bytes = (2 * CS_TN * (NG * 8 + 4) + WAVES * 32 * 64) * sizeof(float) + WAVES * 32 * FM * sizeof(CsPoint);
     // above 64 KiB a kernel has to opt in; once per instantiation and process
     static const int lds_rc = check_hip(
-        hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_candidates_stationary_kernel<NG>),
+        hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_candidates_stationary_kernel<NG, FM>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_bytes),
         "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
     SKM_TRY(lds_rc);
-    const int dbg = getenv("SKM_CS_DBG") ? atoi(getenv("SKM_CS_DBG")) : 0;
-    hipLaunchKernelGGL((gemm_candidates_stationary_kernel<NG>), grid, dim3(CS_THREADS), lds_bytes, ctx->stream, C, k, X, n,
-                       partial_d, ld, xnorm_p, cnorm_p, thr0, cand_count, cand, cap, dbg);
+    hipLaunchKernelGGL((gemm_candidates_stationary_kernel<NG, FM>), grid, dim3(64 * WAVES), lds_bytes, ctx->stream, C, k, X, n,
+                       partial_d, ld, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
     return SKM_OK;
 }
 
 // Whether the register-stationary kernel serves this call; otherwise gemm_candidates_kernel does.
-bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, int n, int partial_d, int64_t ld) {
+bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
+                                       bool whatever_n) {
     const int groups = (partial_d + 7) / 8;
     if (groups > CS_MAX_GROUPS) return false;
     // 16-byte loads of whole groups of 8 columns, rows at least that long
@@ -332,15 +334,15 @@ bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, in
     if ((int64_t) groups * 8 > ld) return false;
     // centroid rows are addressed with 32-bit byte offsets, the tiles requested past the end included
     if (((int64_t) k + 4 * CS_TN) * ld * 4 >= (int64_t(1) << 32)) return false;
-    // a workgroup owns 256 points: below two rounds of workgroups the 128-point kernel fills the chip better
-    return n >= 2 * 512 * CS_POINTS / 2;
+    // a workgroup owns 256 points: below a few rounds of workgroups the 128-point kernel fills the chip better
+    return whatever_n || n >= 512 * CS_POINTS;
 }
 
 int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                                       const float* xnorm_p, const float* cnorm_p, const float* thr0,
                                       uint32_t* cand_count, uint2* cand, uint32_t cap) {
     if (k <= 0 || n <= 0 || partial_d <= 0) return SKM_OK;
-    if (!gemm_candidates_stationary_serves(C, k, X, n, partial_d, ld))
+    if (!gemm_candidates_stationary_serves(C, k, X, n, partial_d, ld, true))
         return set_error(SKM_ERR_INVALID, "register-stationary candidate kernel: unsupported shape");
     // list offsets inside a wavefront's 64 lists are 32-bit
     if ((uint64_t) cap * 64 * sizeof(uint2) >= (uint64_t(1) << 32))
@@ -352,7 +354,9 @@ int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const
         break;
     switch ((partial_d + 7) / 8) {
         SKM_CS_CASE(1) SKM_CS_CASE(2) SKM_CS_CASE(3) SKM_CS_CASE(4) SKM_CS_CASE(5) SKM_CS_CASE(6)
-        SKM_CS_CASE(7) SKM_CS_CASE(8) SKM_CS_CASE(9) SKM_CS_CASE(10) SKM_CS_CASE(11)
+        SKM_CS_CASE(7) SKM_CS_CASE(8) SKM_CS_CASE(9) SKM_CS_CASE(10) SKM_CS_CASE(11) SKM_CS_CASE(12)
+        SKM_CS_CASE(13) SKM_CS_CASE(14) SKM_CS_CASE(15) SKM_CS_CASE(16) SKM_CS_CASE(17) SKM_CS_CASE(18)
+        SKM_CS_CASE(19) SKM_CS_CASE(20)
     }
 #undef SKM_CS_CASE
     return check_hip(hipGetLastError(), "gemm_candidates_stationary_kernel launch");

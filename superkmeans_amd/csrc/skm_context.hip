@@ -195,6 +195,13 @@ int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes) {
     return SKM_OK;
 }
 
+int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(which >= 0 && which <= 2, "which must be 0 (automatic), 1 (tiled) or 2 (register-stationary)");
+    ctx->candidate_kernel = which;
+    return SKM_OK;
+}
+
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr) {
     SKM_REQUIRE(ctx && out_d_ptr, "null argument");
     *out_d_ptr = nullptr;

@@ -28,6 +28,7 @@ struct skm_ctx {
     hipEvent_t copy_done[8] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     unsigned copy_seq = 0;
     size_t workspace_limit = size_t(24) << 30;
+    int candidate_kernel = 0;  // skm_ctx_set_candidate_kernel
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
     void* ws[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t ws_bytes[4] = {0, 0, 0, 0};
@@ -116,7 +117,8 @@ int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, 
                            const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
                            uint2* cand, uint32_t cap);
 // The same for short d' (the points stay in registers); `serves` says whether a call qualifies.
-bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, int n, int partial_d, int64_t ld);
+bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
+                                       bool whatever_n);
 int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                                       const float* xnorm_p, const float* cnorm_p, const float* thr0,
                                       uint32_t* cand_count, uint2* cand, uint32_t cap);

@@ -3,8 +3,9 @@
 //
 // Per chunk of points:
 //   1. seed_distance_kernel     full distance to the previous assignment -> best0, thr0 = best0 * ratios[d']
-//   2. gemm_candidates_kernel   MFMA partial distances; the epilogue emits only pairs below thr0 into
-//                               per-point lists (nothing dense is written)
+//   2. gemm_candidates_kernel or gemm_candidates_stationary_kernel (d' up to 160 and enough points to fill the
+//                               chip with 256-point workgroups): MFMA partial distances; the epilogue emits only
+//                               pairs below thr0 into per-point lists (nothing dense is written)
 //   3. prune_list_kernel        exact per-batch thresholds, block-wise pruning, best candidate
 // After the last chunk, the points whose list overflowed (loose seeds, points with no centroid nearby)
 // are gathered and redone with the dense pair gemm_store_kernel + prune_kernel: same results, more
@@ -12,8 +13,6 @@
 #include "skm_internal.h"
 
 #include <algorithm>
-#include <cstdlib>
-#include <cstdio>
 #include <vector>
 
 namespace skm {
@@ -113,19 +112,15 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         }
         {
             ScopedStage st(ctx, "search/blas");
-            if (gemm_candidates_stationary_serves(d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d) &&
-                !getenv("SKM_CAND_OLD"))
+            if (ctx->candidate_kernel != 1 &&
+                gemm_candidates_stationary_serves(d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d,
+                                                  ctx->candidate_kernel == 2))
                 SKM_TRY(launch_gemm_candidates_stationary(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d,
                                                           d_xnorm_p + i0, d_cnorm_p, d_thr0, d_cand_count,
                                                           (uint2*) ws_cand, cap));
             else
                 SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
                                                d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
-        }
-        if (getenv("SKM_CS_DBG") && (atoi(getenv("SKM_CS_DBG")) & 16)) {
-            double tot = 0;
-            SKM_TRY(reduce_u32_sum_to_host(ctx, d_cand_count, m, &tot));
-            fprintf(stderr, "[dbg] d'=%u candidates emitted: %.0f = %.4f %% of pairs\n", partial_d, tot, 100.0 * tot / ((double) m * k));
         }
         SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over));
         {

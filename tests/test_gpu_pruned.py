@@ -11,7 +11,8 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False):
+def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, kernel=0):
+    """kernel: skm_ctx_set_candidate_kernel (0 automatic, 1 tiled, 2 register-stationary where the shape allows)."""
     n, d = X.shape
     k = C.shape[0]
     H, V = oracle.dimension_split(d)
@@ -25,9 +26,13 @@ def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False):
     idx, dist = ctx.array(np.ascontiguousarray(prev, dtype=np.uint32)), ctx.empty(n)
     total = ctypes.c_uint64()
     stages = (ctypes.c_uint64 * (H // 64 + 2))()
-    capi.check(ctx.lib.skm_assign_pruned(ctx.handle, dX.ptr, n, dC.ptr, dP.ptr, dA.ptr, k, d, V, partial_d, dR.ptr,
-                                         xn.ptr, cn.ptr, idx.ptr, dist.ptr, ctypes.byref(total),
-                                         stages if accounting else None))
+    capi.check(ctx.lib.skm_ctx_set_candidate_kernel(ctx.handle, kernel))
+    try:
+        capi.check(ctx.lib.skm_assign_pruned(ctx.handle, dX.ptr, n, dC.ptr, dP.ptr, dA.ptr, k, d, V, partial_d, dR.ptr,
+                                             xn.ptr, cn.ptr, idx.ptr, dist.ptr, ctypes.byref(total),
+                                             stages if accounting else None))
+    finally:
+        capi.check(ctx.lib.skm_ctx_set_candidate_kernel(ctx.handle, 0))
     out = idx.download(), dist.download(), total.value, np.array(list(stages), dtype=np.uint64)
     for a in (dX, dC, dP, dA, xn, cn, dR, idx, dist):
         a.free()
@@ -81,6 +86,67 @@ def test_pruned_matches_oracle(capi, ctx, oracle, blobs, n, d, k, partial_d):
     # survivors shrink monotonically through the horizontal steps
     hs = gst[1:-1]
     assert np.all(hs[:-1] >= hs[1:])
+
+
+# The register-stationary candidate kernel: every number of 8-column groups with both wavefront shapes (up to 88
+# columns a wavefront owns 64 points, up to 160 it owns 32), d' not a multiple of 8, fewer points than a workgroup
+# owns, point and centroid counts that are not multiples of 64, a d' beyond its range (161: the tiled kernel runs).
+@pytest.mark.parametrize("n,d,k,partial_d", [(700, 128, 300, 8), (1000, 128, 100, 16), (1000, 132, 260, 23),
+                                             (1700, 256, 1500, 32), (900, 256, 321, 40), (1200, 256, 1100, 49),
+                                             (777, 256, 640, 64), (1100, 600, 1030, 77), (1125, 768, 1100, 88),
+                                             (1200, 768, 1100, 89), (1300, 768, 1280, 96), (2600, 1024, 2500, 128),
+                                             (100, 1024, 60, 103), (1100, 1024, 1088, 160), (300, 1024, 300, 161),
+                                             (131, 512, 63, 72)])
+def test_both_candidate_kernels_give_the_same_bits(capi, ctx, oracle, blobs, n, d, k, partial_d):
+    X, C, prev = _setup(oracle, blobs, n, d, k, seed=n + d + partial_d)
+    ratios = oracle.ratios(d, 1.5)
+    tiled = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=True, kernel=1)
+    stationary = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=True, kernel=2)
+    assert np.array_equal(tiled[0], stationary[0])
+    assert np.array_equal(tiled[1].view(np.uint32), stationary[1].view(np.uint32))
+    assert tiled[2] == stationary[2]
+    assert np.array_equal(tiled[3], stationary[3])
+    oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, partial_d, ratios)
+    bi, bbest, bsecond = oracle.brute_force(X, C)
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    gi = stationary[0]
+    for i in np.nonzero(gi != oi)[0]:
+        assert gi[i] == bi[i] or tie[i], f"point {i}: gpu {gi[i]} oracle {oi[i]} brute {bi[i]}"
+    assert np.sum(gi != oi) <= max(1, int(1e-4 * n))
+
+
+def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs):
+    """Random seeds at k > 1024: thresholds are loose, many points collect more candidates than their list holds
+    (cap = 1024 slots) and are redone densely; the two kernels must still agree bit for bit."""
+    n, d, k = 3000, 256, 2600
+    X, C, _ = _setup(oracle, blobs, n, d, k, seed=11)
+    prev = np.random.default_rng(3).integers(0, k, n).astype(np.uint32)
+    ratios = np.minimum(1.0, 3.0 * oracle.ratios(d, 1.5)).astype(np.float32)  # looser still: most lists overflow
+    ratios[d] = 1.0
+    tiled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=1)
+    stationary = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=2)
+    assert np.array_equal(tiled[0], stationary[0])
+    assert np.array_equal(tiled[1].view(np.uint32), stationary[1].view(np.uint32))
+    assert tiled[2] == stationary[2]
+    oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, 40, ratios)
+    assert np.mean(stationary[0] == oi) >= 0.9999
+
+
+def test_automatic_choice_of_the_candidate_kernel_at_many_points(capi, ctx, oracle, blobs):
+    """131,072 points and more select the register-stationary kernel by themselves; checked against the oracle."""
+    n, d, k, partial_d = 140000, 128, 1100, 32
+    X, C, prev = _setup(oracle, blobs, n, d, k, seed=9)
+    ratios = oracle.ratios(d, 1.5)
+    auto = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios)
+    tiled = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, kernel=1)
+    assert np.array_equal(auto[0], tiled[0]) and np.array_equal(auto[1].view(np.uint32), tiled[1].view(np.uint32))
+    assert auto[2] == tiled[2]
+    oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, partial_d, ratios)
+    bi, bbest, bsecond = oracle.brute_force(X, C)
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    mism = np.nonzero(auto[0] != oi)[0]
+    assert all(auto[0][i] == bi[i] or tie[i] for i in mism)
+    assert len(mism) <= int(1e-4 * n)
 
 
 def test_pruned_with_unit_ratios_is_exact(capi, ctx, oracle, blobs):
