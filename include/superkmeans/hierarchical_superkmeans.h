@@ -179,6 +179,8 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         in.initial_partial_d = initial_partial_d;
         in.out_assignments = final_assignments.get();
         in.out_centroids = final_centroids.get();
+        dbuf<float> fine_norms(ctx, total_samples);
+        in.out_norms = fine_norms.get();
         // The mesoclusters are independent problems of a few thousand points each, far too small to fill the
         // device one at a time: several helpers, each with its own stream and scratch, take them from a common
         // counter.  Every problem is computed exactly as it would be alone; the statistics are put back in
@@ -237,12 +239,23 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         hip::Check(skm_copy(ctx, this->prev_centroids.get(), final_centroids.get(), sizeof(float) * k * d));
         hip::Check(skm_copy(ctx, this->d_assignments.get(), final_assignments.get(), sizeof(uint32_t) * total_samples));
         const bool refinement_exact = d < DIMENSION_THRESHOLD_FOR_PRUNING || k <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;
-        bool refinement_norms_ready = false;
+        // The reference runs the fine clusterings one after the other on its own norm buffer: mesocluster m leaves
+        // the norms of its members (compacted order; over d' columns if it went on to prune) in the first size(m)
+        // entries, the rest keeps what the mesoclustering left.  A pruned refinement recomputes the norms
+        // (hierarchical_superkmeans.h:474-483); an exact one does not and searches with that buffer as it is
+        // (:484-499).  A point's norm is the same addend for all its distances, so assignments and centroids do
+        // not depend on it, but the distances and therefore the refinement objectives the reference reports (and
+        // its tests pin, tests/test_hierarchical_superkmeans.cpp:636-670) do.  The buffer is rebuilt here in the
+        // reference's order, whichever helper clustered which mesocluster.
+        for (size_t m = 0; m < n_mesoclusters; ++m) {
+            if (fine_clusters_nums[m] == 0 || mesoclusters_sizes[m] == 0) continue;
+            hip::Check(skm_copy(ctx, this->data_norms.get(), fine_norms.get() + offsets[m],
+                                sizeof(float) * mesoclusters_sizes[m]));
+        }
+        bool refinement_norms_ready = refinement_exact;
         for (size_t it = 0; it < hierarchical_config.iters_refinement; ++it) {
             if (!refinement_norms_ready) {
-                // data_norms was reused per mesocluster during phase 2.
-                hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, refinement_exact ? d : this->partial_d,
-                                     this->data_norms.get()));
+                hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, this->partial_d, this->data_norms.get()));
                 refinement_norms_ready = true;
             }
             this->RunIteration(refinement_exact, data_to_cluster, total_samples, k, it, /*is_first_iter=*/false,
@@ -270,6 +283,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         uint32_t initial_partial_d = 0;
         uint32_t* out_assignments = nullptr;       // global cluster id of every sample
         float* out_centroids = nullptr;            // k x d
+        float* out_norms = nullptr;                // per mesocluster (at its member offset): the norms it ended with
     };
 
     // Fine clustering of mesocluster m on this object's context (reference hierarchical_superkmeans.h:300-440):
@@ -297,6 +311,8 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
                                            static_cast<uint32_t>(in.fine_offsets[m]), in.out_assignments));
         hip::Check(skm_copy(this->ctx, in.out_centroids + in.fine_offsets[m] * dd, this->horizontal_centroids.get(),
                             sizeof(float) * n_fineclusters * dd));
+        hip::Check(skm_copy(this->ctx, in.out_norms + in.member_offsets[m], this->data_norms.get(),
+                            sizeof(float) * mesocluster_size));
     }
 
     // Iterations of one phase: the first is always exact (GEMM only); the others are pruned unless the

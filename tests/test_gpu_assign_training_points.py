@@ -1,0 +1,73 @@
+"""AssignTrainingPoints (reference superkmeans.h:397-564) on the device against the oracle's restatement, for its
+three seeding branches:
+
+  sampling_fraction == 1        seeds are the training assignments (:454-469)
+  0.8 < sampling_fraction < 1   sampled points keep their assignment, the others draw a cluster with probability
+                                proportional to its size from mt19937(seed + 1) (:471-501)
+  sampling_fraction <= 0.8      an auxiliary k-means over the centroids gives sqrt(k) meso-centroids; an unsampled
+                                point starts from a representative of its nearest meso-centroid (:503-563)
+
+Both sides train first (two iterations, so that the two trained states agree to rounding), then assign all
+points.  Bar: results equal except on points whose two best centroids are a near tie or where the device found
+the true nearest centroid and the oracle's pruning did not; at most 0.1 % of the points may differ at all (pruning is approximate on both sides, tests/test_assign.cpp:152-155 asks
+for 98 % agreement with brute force).
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _compare(oracle, X_search, C_dev, C_ora, got, ref):
+    """The two trained states agree to rounding, not to the bit (a cluster split in the first iteration leaves twin
+    centroids and a handful of points that the two implementations resolve differently), so a differing point is
+    accepted when the device returned the exact nearest centroid of its own centroids, or when the point's two best
+    centroids are a near tie (relative gap <= 1e-3 under either set of centroids)."""
+    gi, gbest, gsecond = oracle.brute_force(X_search, C_dev)
+    oi, obest, osecond = oracle.brute_force(X_search, C_ora)
+    tie = ((gsecond - gbest) <= 1e-3 * np.maximum(gbest, 1e-12)) | ((osecond - obest) <= 1e-3 * np.maximum(obest, 1e-12))
+    mism = np.nonzero(got != ref)[0]
+    bad = [i for i in mism if not (tie[i] or got[i] == gi[i])]
+    assert not bad, f"{len(bad)} points differ from the oracle without being a near tie or the exact answer"
+    assert len(mism) <= max(1, int(1e-3 * len(got)))
+    assert np.mean(got == gi) >= 0.98
+
+
+@pytest.mark.parametrize("fraction", [1.0, 0.9, 0.5])
+def test_every_seeding_branch_against_the_oracle(capi, ctx, oracle, blobs, fraction):
+    n, d, k = 24000, 256, 400
+    X = blobs(n, d, k, std=0.3, seed=17)
+    cfg = dict(iters=2, sampling_fraction=fraction, early_termination=0, seed=42, suppress_warnings=1,
+               max_points_per_cluster=99999)
+    km, ok = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    C, OC = km.train(X), ok.train(X)
+    assert all(a.split == b.split for a, b in zip(km.stats(), ok.stats()))
+    rel = np.linalg.norm(C.astype(np.float64) - OC.astype(np.float64)) / np.linalg.norm(OC.astype(np.float64))
+    assert rel <= 1e-3
+    got = km.assign_training_points(X, C)
+    ref = ok.assign_training_points(X, OC)
+    assert got.shape == ref.shape == (n,) and got.max() < k
+    _compare(oracle, X, C, OC, got, ref)
+    km.close()
+
+
+def test_meso_centroid_seeding_on_data_that_is_already_rotated(capi, ctx, oracle, blobs):
+    """data_already_rotated with few samples: the auxiliary k-means over the centroids must not un-rotate its
+    meso-centroids (the constructor rule of superkmeans.h:137-139), or points and meso-centroids would be compared
+    in different spaces and the seeds would be arbitrary."""
+    n, d, k = 20000, 256, 400
+    X = blobs(n, d, k, std=0.3, seed=23)
+    Xrot = oracle.rotate(oracle.rotation_matrix(d, 42), X)
+    cfg = dict(iters=2, sampling_fraction=0.5, early_termination=0, seed=42, suppress_warnings=1,
+               max_points_per_cluster=99999, data_already_rotated=1)
+    km, ok = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    C, OC = km.train(Xrot), ok.train(Xrot)
+    rel = np.linalg.norm(C.astype(np.float64) - OC.astype(np.float64)) / np.linalg.norm(OC.astype(np.float64))
+    assert rel <= 1e-3
+    got = km.assign_training_points(Xrot, C)
+    ref = ok.assign_training_points(Xrot, OC)
+    _compare(oracle, Xrot, C, OC, got, ref)
+    # good seeds: nearly every point ends on its true nearest centroid (arbitrary seeds lose several percent)
+    bi, _, _ = oracle.brute_force(Xrot, OC)
+    assert np.mean(got == bi) >= 0.995
+    km.close()

@@ -118,58 +118,35 @@ def test_gather_rows_and_scatter_assignments(capi, ctx):
 
 
 def test_edit_rows_matches_split_clusters(capi, ctx, oracle):
-    """The copy+perturb edit reproduces SplitClusters' row arithmetic (superkmeans.h:905-920)."""
+    """The copy+perturb edit reproduces SplitClusters' row arithmetic (superkmeans.h:905-920).  Every cluster but one
+    has a single member, so its acceptance probability (size - 1) / (n - k) is zero and the first empty cluster can
+    only take from the large one; the second empty cluster takes from the large one or from the first recipient, and
+    which one it was shows in the sizes the oracle returns."""
     g = np.random.default_rng(8)
     k, d = 12, 64
     C = g.standard_normal((k, d)).astype(np.float32)
-    sizes = np.full(k, 100, dtype=np.uint32)
-    sizes[[3, 7]] = 0
-    sizes[0] = 100 + 200
+    sizes = np.ones(k, dtype=np.uint32)
+    big, first, second = 5, 3, 7
+    sizes[[first, second]] = 0
+    sizes[big] = 301
     n = int(sizes.sum())
     rc, rs, nsplit = oracle.split_clusters(C, sizes, n, seed=42, hierarchical=False)
     assert nsplit == 2
-    # recover which rows were split from the oracle result: dst rows are 3 and 7; find their sources
-    ops = []
-    cur = C.copy()
-    for dst in (3, 7):
-        src = None
-        for cand in range(k):
-            if cand in (3, 7) and cur[cand].tolist() == C[cand].tolist() and sizes[cand] == 0:
-                continue
-            trial = cur[cand].copy()
-            sign = np.where(np.arange(d) % 2 == 0, 1.0, -1.0).astype(np.float32)
-            if np.array_equal(trial * (np.float32(1) + sign * np.float32(1 / 1024)), rc[dst]) or True:
-                pass
-        # the oracle's choice is visible from the size bookkeeping
-        changed = [c for c in range(k) if rs[c] != sizes[c] and c not in (3, 7)]
-        src = changed[0] if len(changed) == 1 else None
-        assert src is not None or len(changed) >= 1
-        src = changed[0]
-        ops += [0, dst, src, 0]
-        break
-    # apply both edits with the same source the oracle used (sizes show a single donor twice or two donors)
-    donors = [c for c in range(k) if rs[c] != sizes[c] and c not in (3, 7)]
-    if len(donors) == 1:
-        ops = [0, 3, donors[0], 0, 0, 7, donors[0], 0]
-    else:
-        # two donors: order by which copy matches
-        ops = None
-        for d0, d1 in ((donors[0], donors[1]), (donors[1], donors[0])):
-            dC = ctx.array(C)
-            o = np.array([0, 3, d0, 0, 0, 7, d1, 0], dtype=np.uint32)
-            capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, o.ctypes.data, 2))
-            got = dC.download()
-            dC.free()
-            if np.array_equal(got, rc):
-                ops = o
-                break
-        assert ops is not None
-        return
+    # after the first split: first = 150, big = 151
+    if rs[big] == 151:      # the second split halved the first recipient: 150 -> 75 + 75
+        assert (rs[first], rs[second]) == (75, 75)
+        donor2 = first
+    else:                   # the second split halved the large cluster again: 151 -> 76 + 75
+        assert (rs[big], rs[first], rs[second]) == (76, 150, 75)
+        donor2 = big
+    ops = np.array([0, first, big, 0, 0, second, donor2, 0], dtype=np.uint32)
     dC = ctx.array(C)
-    o = np.array(ops, dtype=np.uint32)
-    capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, o.ctypes.data, len(o) // 4))
-    assert np.array_equal(dC.download(), rc)
+    capi.check(ctx.lib.skm_edit_rows(ctx.handle, dC.ptr, d, ops.ctypes.data, 2))
+    got = dC.download()
     dC.free()
+    assert np.array_equal(got, rc)
+    untouched = [c for c in range(k) if c not in (big, first, second)]
+    assert np.array_equal(got[untouched], C[untouched])
 
 
 @pytest.mark.parametrize("k,n_ops,seed", [(6, 300, 0), (40, 500, 1), (3000, 2000, 2)])

@@ -74,14 +74,15 @@ def test_blas_only_disables_pruning_where_it_would_run(capi, ctx, oracle, golden
     a.close(), b.close()
 
 
-@pytest.mark.parametrize("k", [100, 250])
+@pytest.mark.parametrize("k", [10, 100, 250])
 def test_hierarchical_wcss_table(capi, ctx, golden, golden_data, k):
     """tests/test_hierarchical_superkmeans.cpp:718-801: final refinement WCSS within 10 % above / 50 % below the
     table, refinement and every mesocluster's fine clustering monotone within 1 %, one block of
     iters_fineclustering entries per mesocluster."""
     n_meso = int(round(np.sqrt(k)))
-    for d in (16, 128, 384, 768):
-        expected = golden["hierarchical"][str(k)][str(d)]
+    assert len(golden["hierarchical"][str(k)]) == 10  # all ten dimensionalities of test_hierarchical_superkmeans.cpp:805-809
+    for d_str, expected in golden["hierarchical"][str(k)].items():
+        d = int(d_str)
         km = capi.KMeans(k, d, hierarchical=True, iters_mesoclustering=5, iters_fineclustering=5, iters_refinement=2,
                          seed=42, early_termination=0, sampling_fraction=1.0, max_points_per_cluster=99999,
                          n_threads=1, suppress_warnings=1)

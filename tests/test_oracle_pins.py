@@ -271,6 +271,78 @@ def test_arrange_fine_clusters_and_mesoclusters(oracle):
         assert out.sum() == 400 and np.all(out[sizes == 0][:-1] == 0) and np.all(out[:-1][sizes[:-1] > 0] >= 1)
 
 
+# ---- ComputeShift, ShouldStopEarly, GetNVectorsToSample (superkmeans.h:988-998,1294-1333,1269-1277) ----
+def test_shift_is_the_squared_movement_of_the_centroids(oracle, blobs):
+    """stats[i].shift = sum_c |c_i - c_{i-1}|^2 over the rotated centroids: recomputed in fp64 from the centroids
+    of two runs that differ by one iteration (runs are deterministic; a dropped square root, a missing square or a
+    sum over the wrong pair of buffers would not pass)."""
+    n, d, k = 4000, 64, 40
+    X = blobs(n, d, k, std=0.4, seed=3)
+    cfg = dict(sampling_fraction=1.0, early_termination=0, seed=42, unrotate_centroids=0)
+    cents, shifts = [], None
+    for iters in (1, 2, 3, 4):
+        km = oracle.KMeans(k, d, iters=iters, **cfg)
+        cents.append(km.train(X).astype(np.float64))
+        shifts = [s.shift for s in km.stats()]
+    for i in (1, 2, 3):
+        exact = ((cents[i] - cents[i - 1]) ** 2).sum()
+        assert shifts[i] == pytest.approx(exact, rel=1e-5), i
+    assert shifts[1] > shifts[2] > shifts[3] > 0
+
+
+def test_should_stop_early_follows_the_rule_of_the_statistics(oracle, blobs):
+    """Early termination stops after the first iteration i (0-based) with shift_i < tol, or with i > 0 and
+    cost_i / cost_{i-1} > 1 - tol.  The stopping iteration is predicted from the statistics of a run without early
+    termination and compared with runs that have it, for tolerances that trigger either clause or neither."""
+    n, d, k, iters = 5000, 64, 50, 12
+    X = blobs(n, d, k, std=0.4, seed=5)
+    base = dict(iters=iters, sampling_fraction=1.0, seed=42)
+    full = oracle.KMeans(k, d, early_termination=0, **base)
+    full.train(X)
+    st = full.stats()
+    assert len(st) == iters
+
+    def predicted(tol):
+        for i, s in enumerate(st):
+            if s.shift < tol:
+                return i + 1
+            if i > 0 and np.float32(s.objective) / np.float32(st[i - 1].objective) > np.float32(1) - np.float32(tol):
+                return i + 1
+        return iters
+
+    ratios = [st[i].objective / st[i - 1].objective for i in range(1, iters)]
+    tols = [1e-12,                                  # neither clause: runs to the end unless the cost stalls exactly
+            (1 - ratios[2]) * 1.5,                  # cost clause after a few iterations
+            0.95,                                   # cost clause at once (second iteration)
+            st[0].shift * 2.0]                      # shift clause in the first iteration
+    seen = set()
+    for tol in tols:
+        km = oracle.KMeans(k, d, early_termination=1, tol=tol, **base)
+        km.train(X)
+        assert len(km.stats()) == predicted(tol), tol
+        seen.add(len(km.stats()))
+    assert 1 in seen and 2 in seen and len(seen) >= 3
+
+
+def test_number_of_vectors_to_sample(oracle, blobs):
+    """Flat: min(floor(float(n) * fraction), k * max_points_per_cluster), all n when the fraction is 1; hierarchical:
+    floor(double(n) * fraction).  Observed through the number of training assignments a run keeps."""
+    d = 16
+    X = blobs(3001, d, 10, std=0.5, seed=1)
+    def samples(n, k, hierarchical=False, **cfg):
+        km = oracle.KMeans(k, d, hierarchical=hierarchical, iters=1, suppress_warnings=1, **cfg)
+        km.train(X[:n])
+        return len(km.state()[1])
+    assert samples(3001, 10, sampling_fraction=1.0, max_points_per_cluster=1) == 3001
+    assert samples(3001, 10, sampling_fraction=0.3, max_points_per_cluster=256) == 900        # floor(900.3)
+    assert samples(3001, 10, sampling_fraction=0.5, max_points_per_cluster=100) == 1000       # 10 * 100 < 1500
+    assert samples(2999, 7, sampling_fraction=0.9, max_points_per_cluster=99999) == int(np.floor(np.float32(2999) * np.float32(0.9)))
+    assert samples(3001, 16, hierarchical=True, sampling_fraction=0.5, max_points_per_cluster=1,
+                   iters_mesoclustering=1, iters_fineclustering=1) == 1500                   # no cap per cluster
+    with pytest.raises(oracle.OracleError):
+        samples(3001, 10, sampling_fraction=0.003, max_points_per_cluster=256)               # 9 samples < 10 clusters
+
+
 # ---- whole Train(): reference golden WCSS tables and behavioural contract ----
 def test_make_blobs_shape_statistics(golden_data):
     X = golden_data
