@@ -14,7 +14,14 @@ The CPU baseline is
 the CPU oracle (OpenMP + BLAS restatement of the reference path) on a bounded prefix of the same
 points, on the host cores of the same box.
 
-Prints one JSON line.  Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N --d D --k K]
+--config selects one of the five benchmark configurations (default C2, the headline; its JSON line keeps the same
+keys): C1 n=100,000 d=768 k=1,000 (25 iterations), C2, C3 n=10,000,000 d=1024 k=10,000 (Assign only), C4 hierarchical
+n=10,000,000 d=1024 k=65,536, C5 n=2,000,000 d=1536 k=4,096 (low intrinsic dimension, heavy tails).  Every
+configuration reports Assign points/s, Train seconds end to end and per iteration, the stage table and the CPU
+baseline on a bounded sample; the transfer-inclusive leg runs by default where the host copy of the points is at most
+16 GB (C1, C2, C5) and on request (--host-pointers) for the 41 GB configurations.
+
+Prints one JSON line.  Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2] [--n N --d D --k K]
 """
 import argparse
 import json
@@ -38,24 +45,56 @@ PEAK_HBM_GBPS = 8000.0
 MEASURED_TRAFFIC_BYTES = {
     (1_000_000, 1024, 10_000): int(((31_523_194 + 2_005_616) * 1.943 + 609_375 + 7_812) * 1024),
 }
+# The same counters summed over the seed, list-walk and overflow kernels of one Train of (n, d, k, iterations); recorded
+# from the profile named in profiles/ for that shape, null where none was taken.
+MEASURED_PRUNE_TRAFFIC_BYTES = {}
+
+
+# name -> (n, d, k, Train iterations, hierarchical, description of the generator)
+CONFIGS = {
+    "C1": (100_000, 768, 1_000, 25, False, "1,000 centres ~ N(0, I), point = centre + 0.3 N(0, I)"),
+    "C2": (1_000_000, 1024, 10_000, 10, False, "seeded Gaussian mixture with 1/sqrt(j+1) variance decay"),
+    "C3": (10_000_000, 1024, 10_000, 0, False, "fixed centroids ~ N(0, I) normalised, point = centroid + 0.5 N(0, I)"),
+    "C4": (10_000_000, 1024, 65_536, 0, True, "two-level mixture: 256 coarse centres, 65,536 fine centres at sigma 0.2, "
+                                               "point noise 0.1"),
+    "C5": (2_000_000, 1536, 4_096, 10, False, "rank-64 Gaussian latent through a fixed linear map + Student-t(3) noise"),
+}
+
+
+def generate_points(_capi, lib, ctx, name, dX, n, d, k):
+    """Fills dX (n x d, device) with the configuration's seeded synthetic rows (L2-normalised)."""
+    if name == "C1":
+        _capi.check(lib.skm_synth_gaussian_mixture(ctx.handle, dX.ptr, n, d, 0, k, 101, 102, 1.0, 0.3, 0.0, 1))
+    elif name == "C3":
+        _capi.check(lib.skm_synth_gaussian_mixture(ctx.handle, dX.ptr, n, d, 0, k, 77, 78, 1.0, 0.5, 0.0, 1))
+    elif name == "C4":
+        _capi.check(lib.skm_synth_two_level_mixture(ctx.handle, dX.ptr, n, d, 0, 256, 65_536, 9, 0.2, 0.1))
+    elif name == "C5":
+        _capi.check(lib.skm_synth_low_rank(ctx.handle, dX.ptr, n, d, 0, 64, 21, 0.05))
+    else:
+        _capi.check(lib.skm_synth_gaussian_mixture(ctx.handle, dX.ptr, n, d, 0, k, 1234, 5678, 1.0, 0.3, 0.25, 1))
 
 
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--config", choices=sorted(CONFIGS), default="C2")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--n", type=int, default=1_000_000)
-    ap.add_argument("--d", type=int, default=1024)
-    ap.add_argument("--k", type=int, default=10_000)
-    ap.add_argument("--train-iters", type=int, default=10)
+    ap.add_argument("--n", type=int, default=None)
+    ap.add_argument("--d", type=int, default=None)
+    ap.add_argument("--k", type=int, default=None)
+    ap.add_argument("--train-iters", type=int, default=None)
     ap.add_argument("--cpu-assign-points", type=int, default=131072)
     ap.add_argument("--cpu-train-points", type=int, default=65536)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-train", action="store_true")
     ap.add_argument("--host-pointers", action="store_true",
-                    help="also run the transfer-inclusive leg (Assign and Train called with host pointers); off by "
-                         "default so that a kernel trace of the default command holds the resident launches only")
+                    help="run the transfer-inclusive leg (Assign and Train called with host pointers) also where the "
+                         "host copy of the points exceeds 16 GB")
+    ap.add_argument("--no-host-pointers", action="store_true",
+                    help="skip the transfer-inclusive leg, so that a kernel trace of the command holds the resident "
+                         "launches only")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain row-copy kernel of known size (1 GiB read + 1 GiB write) three times; "
                          "used to scale the FETCH_SIZE / WRITE_SIZE hardware counters")
@@ -81,20 +120,27 @@ def main():
         ctx.close()
         return
 
-    n, d, k = args.n, args.d, args.k
-    cfg = dict(iters=args.train_iters, sampling_fraction=1.0, early_termination=0, seed=42, suppress_warnings=1)
-    km = _capi.KMeans(k, d, **cfg)
+    cn, cd, ck, citers, hierarchical, generator = CONFIGS[args.config]
+    n, d, k = args.n or cn, args.d or cd, args.k or ck
+    train_iters = args.train_iters if args.train_iters is not None else citers
+    no_train = args.no_train or (train_iters == 0 and not hierarchical)
+    if hierarchical:
+        cfg = dict(early_termination=0, seed=42, suppress_warnings=1)  # 3 + 5 + 0 iterations, the reference's defaults
+    else:
+        cfg = dict(iters=max(1, train_iters), sampling_fraction=1.0, early_termination=0, seed=42, suppress_warnings=1)
+    km = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
     ctx, lib = km.ctx, km.lib
+    host_leg = not args.no_host_pointers and (args.host_pointers or 4.0 * n * d <= 16e9)
 
     # ---- synthetic points, resident in HBM ----
     dX = ctx.empty((n, d))
-    _capi.check(lib.skm_synth_gaussian_mixture(ctx.handle, dX.ptr, n, d, 0, k, 1234, 5678, 1.0, 0.3, 0.25, 1))
+    generate_points(_capi, lib, ctx, args.config, dX, n, d, k)
     ctx.sync()
 
     # ---- Train (device-resident data), per-stage device timers ----
     train = None
     centroids = None
-    if not args.no_train:
+    if not no_train:
         ctx.prof_enable(True)
         ctx.prof_reset()
         km.set_prune_accounting(False)
@@ -104,24 +150,30 @@ def main():
         train_s = time.perf_counter() - t0
         prof = ctx.prof()
         ctx.prof_enable(False)
-        stats = km.stats()
+        # hierarchical: the owner object's timers cover the mesoclustering and the refinement; the fine clusterings
+        # run on helper objects with their own contexts and show up as the rest of the end-to-end time
+        phase_stats = {name: km.stats(which) for which, name in ((1, "mesoclustering"), (2, "fineclustering"), (3, "refinement"))} \
+            if hierarchical else None
+        stats = (phase_stats["mesoclustering"] + phase_stats["refinement"]) if hierarchical else km.stats()
         n_gemm = sum(1 for s in stats if s.is_gemm_only)
         n_pruned = len(stats) - n_gemm
         ms = lambda name: prof.get(name, (0.0, 0))[0]
         calls = lambda name: prof.get(name, (0.0, 0))[1]
         # A second, untimed Train of an identical object only to count the pairs entering each pruning step.
-        km2 = _capi.KMeans(k, d, **cfg)
-        km2.set_prune_accounting(True)
-        km2.train_device(dX, n)
-        acct = km2.prune_accounting()
-        km2.close()
+        acct = []
+        if n_pruned and not hierarchical:
+            km2 = _capi.KMeans(k, d, **cfg)
+            km2.set_prune_accounting(True)
+            km2.train_device(dX, n)
+            acct = km2.prune_accounting()
+            km2.close()
         _, V = _capi.dimension_split(d)
         prune_bytes = 0.0
         for row, s in zip(acct, [s for s in stats if not s.is_gemm_only]):
             pairs_blocks = float(sum(int(x) for x in row[1:-1]))
             pairs_tail = float(row[-1])
             prune_bytes += 4.0 * (n * (d - s.partial_d) + 64.0 * pairs_blocks + (V - s.partial_d) * pairs_tail) + 8.0 * n
-        partial_flops = sum(2.0 * n * k * s.partial_d for s in stats if not s.is_gemm_only)
+        partial_flops = sum(2.0 * n * k * s.partial_d for s in stats if not s.is_gemm_only)  # flat runs only
         stage = {}
 
         def add_stage(name, bound, work, t_ms, unit_peak):
@@ -132,15 +184,18 @@ def main():
                            "peak": unit_peak, "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
                            "frac": round(ach / unit_peak, 4)}
 
-        add_stage("rotation", "mfma", 2.0 * (n + k) * d * d, ms("rotator"), PEAK_FP32_MFMA_TFLOPS)
-        add_stage("full_distance_gemm", "mfma", 2.0 * n * k * d * n_gemm, ms("search/1st_blas"), PEAK_FP32_MFMA_TFLOPS)
+        # the owner object of a hierarchical Train searches among the sqrt(k) mesocluster centroids
+        ks = int(round(k ** 0.5)) if hierarchical else k
+        add_stage("rotation", "mfma", 2.0 * (n + ks) * d * d, ms("rotator"), PEAK_FP32_MFMA_TFLOPS)
+        add_stage("full_distance_gemm", "mfma", 2.0 * n * ks * d * n_gemm, ms("search/1st_blas"), PEAK_FP32_MFMA_TFLOPS)
         # the dense redo of overflowing points is part of the same two stages
         add_stage("partial_distance_gemm", "mfma", partial_flops, ms("search/blas") + ms("search/overflow/blas"),
                   PEAK_FP32_MFMA_TFLOPS)
         add_stage("prune", "hbm", prune_bytes, ms("search/seed") + ms("search/pdx") + ms("search/overflow/pdx"),
                   PEAK_HBM_GBPS)
-        add_stage("update", "hbm", len(stats) * (4.0 * n * d + 8.0 * n + 4.0 * k * d + 4.0 * k), ms("update_centroids"), PEAK_HBM_GBPS)
-        add_stage("pdx_relayout", "hbm", calls("consolidate/pdxify") * (2.0 * 4 * k * d + 4.0 * k * V), ms("consolidate/pdxify"), PEAK_HBM_GBPS)
+        add_stage("update", "hbm", len(stats) * (4.0 * n * d + 8.0 * n + 4.0 * ks * d + 4.0 * ks), ms("update_centroids"), PEAK_HBM_GBPS)
+        if not hierarchical:
+            add_stage("pdx_relayout", "hbm", calls("consolidate/pdxify") * (2.0 * 4 * k * d + 4.0 * k * V), ms("consolidate/pdxify"), PEAK_HBM_GBPS)
         iter_ms = ms("search") + ms("update_centroids") + ms("consolidate/pdxify") + ms("consolidate/splitting") + \
             ms("compute_cost") + ms("shift") + ms("norms_calc")
         gemm_iter_ms = ms("search/1st_blas") + ms("search/merge")
@@ -156,7 +211,29 @@ def main():
             "not_pruned_pct": [round(s.not_pruned_pct, 5) for s in stats],
             "stages": stage,
         }
+        if n_pruned and "prune" in stage:
+            # the walk of the candidate lists is a chain of dependent 256-byte gathers served mostly by L2 and the
+            # memory-side cache, so besides the algorithmic GB/s: nanoseconds per (pair, 64-dimension block) visited
+            blocks_visited = float(sum(sum(int(x) for x in row[1:-1]) for row in acct))
+            if blocks_visited > 0:
+                stage["prune"]["pair_blocks_visited"] = blocks_visited
+                stage["prune"]["ns_per_pair_block"] = round(stage["prune"]["ms"] * 1e6 / blocks_visited, 4)
+            measured = MEASURED_PRUNE_TRAFFIC_BYTES.get((n, d, k, len(stats)))
+            if measured:
+                stage["prune"]["measured_bytes"] = measured
+                stage["prune"]["measured_frac"] = round(measured / (stage["prune"]["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+        if hierarchical:
+            train["phases"] = {name: {"iterations": len(v), "final_objective": (v[-1].objective if v and name != "fineclustering" else None)}
+                               for name, v in phase_stats.items()}
+            train["owner_device_ms"] = round(iter_ms + ms("rotator"), 2)
+            train["fine_phase_and_host_s"] = round(train_s - (iter_ms + ms("rotator")) * 1e-3, 4)
 
+    if centroids is None and args.config == "C3":
+        # the fixed, seeded centroids of the Assign-only configuration: the generator's own centres
+        dC3 = ctx.empty((k, d))
+        _capi.check(lib.skm_synth_gaussian_mixture(ctx.handle, dC3.ptr, k, d, 0, 0, 0, 79, 0.0, 1.0, 0.0, 1))
+        centroids = dC3.download()
+        dC3.free()
     if centroids is None:
         centroids = dX.download(k)  # first k points as centroids
     dC = ctx.array(centroids)
@@ -193,7 +270,7 @@ def main():
 
     # ---- PCIe-inclusive leg (reported beside `value`, never as it): the same calls on host pointers ----
     host_pointers = None
-    if args.host_pointers:
+    if host_leg:
         Xhost = dX.download()
         km.assign(Xhost[: min(n, 4096)], centroids)  # buffers of the host path touched once
         t0 = time.perf_counter()
@@ -203,8 +280,8 @@ def main():
                          "assign_equals_resident": bool(np.array_equal(host_assign, gpu_assign)),
                          "note": "pageable host rows, uploaded in 256 MiB slabs on a transfer stream while the "
                                  "previous slab is searched"}
-        if not args.no_train:
-            kmh = _capi.KMeans(k, d, **cfg)
+        if not no_train:
+            kmh = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
             t0 = time.perf_counter()
             host_centroids = kmh.train(Xhost)
             host_pointers["train_s_end_to_end"] = round(time.perf_counter() - t0, 4)
@@ -220,19 +297,24 @@ def main():
         O.load()
         O.set_threads(0)
         cores = O.get_threads()
-        m = min(n, args.cpu_assign_points)
+        # a bounded sample: at most the work of 131,072 points against 10,000 centroids of 1,024 dimensions
+        m = max(1024, min(n, args.cpu_assign_points, int(2.7e12 / (2.0 * k * d))))
         Xh = dX.download(m)
         ok = O.KMeans(k, d, sampling_fraction=1.0, suppress_warnings=1)
-        t0 = time.perf_counter()
-        oa = ok.assign(Xh, centroids)
-        cpu_assign_s = time.perf_counter() - t0
+        cpu_assign_s = None
+        for _ in range(2):  # the host share of the box is noisy: the better of two runs
+            t0 = time.perf_counter()
+            oa = ok.assign(Xh, centroids)
+            took = time.perf_counter() - t0
+            cpu_assign_s = took if cpu_assign_s is None else min(cpu_assign_s, took)
         agree = float(np.mean(oa == gpu_assign[:m]))
         cpu = {"value": round(m / cpu_assign_s, 1), "unit": "points/s", "cores": int(cores), "kind": "port",
-               "sample": f"Assign of the first {m} of the {n} points against the same {k} centroids, "
-                         f"{cpu_assign_s:.2f} s, BLAS={os.path.basename(O.blas_name())}",
+               "sample": f"Assign of the first {m} of the {n} points against the same {k} centroids, best of two runs "
+                         f"{cpu_assign_s:.2f} s, oracle built with g++ -O3 -march=x86-64-v3 -fopenmp, "
+                         f"BLAS={os.path.basename(O.blas_name())}",
                "assign_agreement_with_gpu": agree}
         mt = min(n, args.cpu_train_points)
-        if mt >= k and not args.no_train:
+        if mt >= k and not no_train and not hierarchical:
             okt = O.KMeans(k, d, iters=3, sampling_fraction=1.0, early_termination=0, suppress_warnings=1)
             t0 = time.perf_counter()
             okt.train(Xh[:mt] if mt <= m else dX.download(mt))
@@ -254,8 +336,9 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": f"SuperKMeans Assign (+ Train {args.train_iters} iters) fp32, n={n}, d={d}, k={k}, "
-                               "seeded Gaussian mixture with 1/sqrt(j+1) variance decay, rows L2-normalised, resident in HBM"},
+        "config": {"workload": f"{args.config}: {'Hierarchical' if hierarchical else ''}SuperKMeans Assign"
+                               + ("" if no_train else f" (+ Train {'3+5+0' if hierarchical else train_iters} iters)")
+                               + f" fp32, n={n}, d={d}, k={k}, {generator}, rows L2-normalised, resident in HBM"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "train": train,
