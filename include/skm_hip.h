@@ -65,6 +65,11 @@ int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which);
  * superkmeans.h:191-201). */
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr);
 int skm_free(skm_ctx* ctx, void* d_ptr);
+/* Blocks released through skm_free, by a context's workspace or by skm_ctx_destroy are kept per device and handed
+ * out again by later allocations of about the same size (allocating and releasing the multi-gigabyte buffers of a
+ * Train costs milliseconds each time, and a release waits for the whole device).  The cache holds at most 96 GiB or
+ * 2,048 blocks, empties itself when an allocation fails, and is emptied on request by this call. */
+int skm_device_cache_trim(int device);
 int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);
 /* Upload on the context's transfer stream: work queued on the context before the call keeps running during the

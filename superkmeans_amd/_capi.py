@@ -29,6 +29,7 @@ _PROTOTYPES = {
     "skm_ctx_set_candidate_kernel": (c_int, [c_void_p, c_int]),
     "skm_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "skm_free": (c_int, [c_void_p, c_void_p]),
+    "skm_device_cache_trim": (c_int, [c_int]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_upload_overlapped": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_householder_q": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),

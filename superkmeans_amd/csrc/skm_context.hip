@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <unordered_map>
+
 namespace skm {
 
 static thread_local char g_last_error[512] = "";
@@ -23,22 +26,89 @@ int check_hip(hipError_t e, const char* what) {
     return set_error(code, "HIP error %d (%s) in %s", (int) e, hipGetErrorString(e), what);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Device blocks released by skm_free, by a context's workspace or by skm_ctx_destroy are kept and handed out
+// again: hipMalloc / hipFree of the gigabyte-sized buffers of a Train cost milliseconds each and hipFree waits
+// for the whole device.  One cache per device and process; a request takes the smallest cached block of at least
+// its size and at most 1/8 more.  The cache holds at most DEVICE_CACHE_MAX_BYTES and DEVICE_CACHE_MAX_BLOCKS
+// (beyond that a released block goes back to the driver), and is emptied when an allocation fails or on
+// skm_device_cache_trim.  A block enters the cache only after the releasing context's stream has drained.
+// ---------------------------------------------------------------------------------------------
+namespace {
+constexpr size_t DEVICE_CACHE_MAX_BYTES = size_t(96) << 30;
+constexpr size_t DEVICE_CACHE_MAX_BLOCKS = 2048;
+struct DeviceCache {
+    std::mutex lock;
+    std::multimap<size_t, void*> idle;           // size -> block
+    std::unordered_map<void*, size_t> size_of;   // every block handed out or idle
+    size_t idle_bytes = 0;
+};
+DeviceCache& device_cache(int device) {
+    static DeviceCache caches[64];
+    return caches[(device >= 0 && device < 64) ? device : 0];
+}
+void trim_locked(DeviceCache& c) {
+    for (auto& kv : c.idle) {
+        (void) hipFree(kv.second);
+        c.size_of.erase(kv.second);
+    }
+    c.idle.clear();
+    c.idle_bytes = 0;
+}
+} // namespace
+
+int device_alloc(int device, size_t bytes, void** out) {
+    *out = nullptr;
+    if (bytes == 0) bytes = 16;
+    bytes = (bytes + 255) / 256 * 256;
+    DeviceCache& c = device_cache(device);
+    std::lock_guard<std::mutex> guard(c.lock);
+    auto it = c.idle.lower_bound(bytes);
+    if (it != c.idle.end() && it->first <= bytes + bytes / 8) {
+        *out = it->second;
+        c.idle_bytes -= it->first;
+        c.idle.erase(it);
+        return SKM_OK;
+    }
+    hipError_t e = hipMalloc(out, bytes);
+    if (e != hipSuccess) {
+        (void) hipGetLastError();
+        trim_locked(c);
+        e = hipMalloc(out, bytes);
+    }
+    if (e != hipSuccess) return check_hip(e, "hipMalloc");
+    c.size_of[*out] = bytes;
+    return SKM_OK;
+}
+
+// The caller guarantees that no queued work uses the block any more.
+int device_release(int device, void* ptr) {
+    if (!ptr) return SKM_OK;
+    DeviceCache& c = device_cache(device);
+    std::lock_guard<std::mutex> guard(c.lock);
+    const auto known = c.size_of.find(ptr);
+    if (known == c.size_of.end()) return check_hip(hipFree(ptr), "hipFree");  // not one of ours
+    const size_t bytes = known->second;
+    if (c.idle.size() >= DEVICE_CACHE_MAX_BLOCKS || c.idle_bytes + bytes > DEVICE_CACHE_MAX_BYTES) {
+        c.size_of.erase(known);
+        return check_hip(hipFree(ptr), "hipFree");
+    }
+    c.idle.emplace(bytes, ptr);
+    c.idle_bytes += bytes;
+    return SKM_OK;
+}
+
 int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out) {
     if (slot < 0 || slot >= 4) return set_error(SKM_ERR_INVALID, "bad workspace slot");
     if (ctx->ws_bytes[slot] < bytes) {
         if (ctx->ws[slot]) {
             SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-            SKM_HIP_TRY(hipFree(ctx->ws[slot]));
+            SKM_TRY(device_release(ctx->device, ctx->ws[slot]));
             ctx->ws[slot] = nullptr;
             ctx->ws_bytes[slot] = 0;
         }
-        size_t want = bytes + bytes / 8;
-        hipError_t e = hipMalloc(&ctx->ws[slot], want);
-        if (e != hipSuccess) {
-            want = bytes;
-            SKM_HIP_TRY(hipMalloc(&ctx->ws[slot], want));
-        }
-        ctx->ws_bytes[slot] = want;
+        SKM_TRY(device_alloc(ctx->device, bytes, &ctx->ws[slot]));
+        ctx->ws_bytes[slot] = bytes;
     }
     *out = ctx->ws[slot];
     return SKM_OK;
@@ -169,7 +239,7 @@ int skm_ctx_destroy(skm_ctx* ctx) {
     }
     for (auto e : ctx->event_pool) (void) hipEventDestroy(e);
     for (int i = 0; i < 4; ++i)
-        if (ctx->ws[i]) (void) hipFree(ctx->ws[i]);
+        if (ctx->ws[i]) (void) device_release(ctx->device, ctx->ws[i]);
     if (ctx->h_pinned) (void) hipHostFree(ctx->h_pinned);
     if (ctx->copy_stream) {
         (void) hipStreamSynchronize(ctx->copy_stream);
@@ -204,10 +274,18 @@ int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which) {
 
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr) {
     SKM_REQUIRE(ctx && out_d_ptr, "null argument");
-    *out_d_ptr = nullptr;
-    if (bytes == 0) bytes = 16;
     SKM_HIP_TRY(hipSetDevice(ctx->device));
-    SKM_HIP_TRY(hipMalloc(out_d_ptr, bytes));
+    return device_alloc(ctx->device, bytes, out_d_ptr);
+}
+
+int skm_device_cache_trim(int device) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n)
+        return set_error(SKM_ERR_INVALID, "skm_device_cache_trim: no such device");
+    SKM_HIP_TRY(hipSetDevice(device));
+    DeviceCache& c = device_cache(device);
+    std::lock_guard<std::mutex> guard(c.lock);
+    trim_locked(c);
     return SKM_OK;
 }
 
@@ -215,8 +293,8 @@ int skm_free(skm_ctx* ctx, void* d_ptr) {
     SKM_REQUIRE(ctx, "null context");
     if (!d_ptr) return SKM_OK;
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-    SKM_HIP_TRY(hipFree(d_ptr));
-    return SKM_OK;
+    if (ctx->copy_stream) SKM_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
+    return device_release(ctx->device, d_ptr);
 }
 
 int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {

@@ -65,6 +65,10 @@ int check_hip(hipError_t e, const char* what);
         if (!(cond)) return ::skm::set_error(SKM_ERR_INVALID, "%s: %s", __func__, msg);           \
     } while (0)
 
+// Device blocks through the per-device cache of released blocks (skm_context.hip).
+int device_alloc(int device, size_t bytes, void** out);
+int device_release(int device, void* ptr);
+
 // Returns a scratch buffer of at least `bytes` for slot `slot` (grow-only).
 int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out);
 int pinned(skm_ctx* ctx, size_t bytes, void** out);
