@@ -59,11 +59,34 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+// Which point a wavefront takes.  Workgroups go to the eight compute dies in turn (workgroup b runs on die b % 8, each
+// with its own L2), so the grid is read as eight contiguous ranges of slots, one per die: consecutive slots, which
+// under a cluster order hold points that gather the same centroid rows and blocks, stay on one die.  The launch has
+// 8 * ceil(workgroups / 8) workgroups; a slot past the end returns -1.
+__device__ __forceinline__ int point_of_wave(const uint32_t* __restrict__ order, int n, int waves_per_group) {
+    const int per_die = (int) (gridDim.x / 8);
+    const int group = (int) (blockIdx.x % 8) * per_die + (int) (blockIdx.x / 8);
+    const int slot = group * waves_per_group + (int) (threadIdx.x >> 6);
+    if (slot >= n) return -1;
+    return order ? (int) order[slot] : slot;
+}
+inline unsigned die_striped_groups(int n, int waves_per_group) {
+    const unsigned groups = (unsigned) ((n + waves_per_group - 1) / waves_per_group);
+    return (groups + 7) / 8 * 8;
+}
+
 // Four consecutive floats of a point row (16-byte load when rows are aligned).
 template <bool VEC>
 __device__ __forceinline__ float4 load_x4(const float* p) {
     if (VEC) return *reinterpret_cast<const float4*>(p);
     return make_float4(p[0], p[1], p[2], p[3]);
+}
+
+// The same for data that is read once per launch: a non-temporal load, which leaves the caches to the centroids.
+__device__ __forceinline__ float4 load_once4(const float* p) {
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
+    return make_float4(v.x, v.y, v.z, v.w);
 }
 
 // Keeps the survivors whose accumulated distance is below thr, preserving order. In-place: slot s
@@ -279,11 +302,12 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
 template <bool VEC>
 __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
     const float* __restrict__ x, const float* __restrict__ c, const uint32_t* __restrict__ idx, int n, int d,
-    const float* __restrict__ ratios, int partial_d, float* __restrict__ best0, float* __restrict__ thr0
+    const float* __restrict__ ratios, int partial_d, float* __restrict__ best0, float* __restrict__ thr0,
+    const uint32_t* __restrict__ order
 ) {
     const int lane = threadIdx.x & 63;
-    const int p = blockIdx.x * PRUNE_WAVES + (threadIdx.x >> 6);
-    if (p >= n) return;
+    const int p = point_of_wave(order, n, PRUNE_WAVES);
+    if (p < 0) return;
     const float* xq = x + (int64_t) p * d;
     const float* cp = c + (int64_t) idx[p] * d;
     float s = 0.0f;
@@ -294,7 +318,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
             float4 xv[4], cv[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                xv[u] = *reinterpret_cast<const float4*>(xq + t + 256 * u);
+                xv[u] = load_once4(xq + t + 256 * u);
                 cv[u] = *reinterpret_cast<const float4*>(cp + t + 256 * u);
             }
 #pragma unroll
@@ -307,7 +331,7 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
             }
         }
         for (; t < d; t += 256) {
-            const float4 xv = *reinterpret_cast<const float4*>(xq + t);
+            const float4 xv = load_once4(xq + t);
             const float4 cv = *reinterpret_cast<const float4*>(cp + t);
             float e;
             e = cv.x - xv.x; s += e * e;
@@ -350,6 +374,7 @@ struct PruneListArgs {
     float* dist;
     uint32_t* not_pruned;
     unsigned long long* stage_pairs;
+    const uint32_t* order;        // null, or the sequence in which the wavefronts take the points
     int n, k, d, vertical_d, partial_d;
 };
 
@@ -360,8 +385,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     __shared__ float s_parts[PRUNE_WAVES][16 * 8];  // [block of the group][survivor]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int p = blockIdx.x * PRUNE_WAVES + wave;
-    if (p >= a.n) return;
+    const int p = point_of_wave(a.order, a.n, PRUNE_WAVES);
+    if (p < 0) return;
     float* parts = s_parts[wave];
     const uint32_t n_cand = a.cand_count[p];
     if (n_cand > a.cap) return;  // handled densely by the caller
@@ -602,28 +627,29 @@ __global__ __launch_bounds__(256) void scatter_u32_kernel(const uint32_t* __rest
 }
 
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
-                         const float* ratios, int partial_d, float* best0, float* thr0) {
+                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order) {
     if (n <= 0) return SKM_OK;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(c) % 16 == 0);
-    dim3 grid((n + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    dim3 grid(die_striped_groups(n, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (vec)
-        hipLaunchKernelGGL(seed_distance_kernel<true>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0);
+        hipLaunchKernelGGL(seed_distance_kernel<true>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order);
     else
-        hipLaunchKernelGGL(seed_distance_kernel<false>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0);
+        hipLaunchKernelGGL(seed_distance_kernel<false>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order);
     return check_hip(hipGetLastError(), "seed_distance_kernel launch");
 }
 
 int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
-                      unsigned long long* d_stage_pairs) {
+                      unsigned long long* d_stage_pairs, const uint32_t* order) {
     if (n_chunk <= 0) return SKM_OK;
     PruneListArgs a;
+    a.order = order;
     a.cand = cand; a.cand_count = cand_count; a.cap = cap; a.best0 = best0; a.x = x; a.pdx = pdx; a.aux = aux;
     a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
-    dim3 grid((n_chunk + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    dim3 grid(die_striped_groups(n_chunk, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (vec && d_stage_pairs)
         hipLaunchKernelGGL((prune_list_kernel<true, true>), grid, block, 0, ctx->stream, a);
     else if (vec)

@@ -16,42 +16,37 @@
 namespace skm {
 
 constexpr int SORT_THREADS = 256;
-constexpr int SORT_TILE = 4096;  // elements per workgroup and pass
+// Elements per workgroup and pass.  Smaller tiles give more workgroups but shorter runs of equal digits per tile: at
+// 1,024 the scatter of a pass over random low digits writes 16-byte runs and takes longer than at 4,096.
+constexpr int SORT_TILE = 4096;
 constexpr int RADIX = 256;
 
-// Exclusive scan of `len` counters by one workgroup (len is 256 * n_tiles: a few hundred KB at most).
-// Each of the 16 wavefronts owns a contiguous segment: it adds the segment up with coalesced loads, the 16
-// totals are exchanged through LDS (the only barrier), then the wavefront scans its segment 64 counters at a
-// time with shuffles, carrying the running total in a register.
-__global__ __launch_bounds__(1024) void exclusive_scan_kernel(
-    const uint32_t* __restrict__ in, uint32_t* __restrict__ out, size_t len
+// Second step of a radix pass.  The histograms are stored digit-major, so the global base of a (digit, tile) pair is
+// (sum of all smaller digits) + (sum of the same digit over the earlier tiles).  One wavefront per digit scans its own
+// row of tile counts, 64 at a time with shuffles and a running carry, and leaves the digit's total; the scatter
+// kernel adds the 256 totals up by itself.  The 256 rows are scanned side by side instead of one scan over
+// 256 * n_tiles counters by a single workgroup.
+__global__ __launch_bounds__(64) void digit_rows_scan_kernel(
+    const uint32_t* __restrict__ hist, uint32_t n_tiles, uint32_t* __restrict__ bases, uint32_t* __restrict__ totals
 ) {
-    __shared__ uint32_t s_wave[16];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const size_t seg = ((len + 15) / 16 + 63) / 64 * 64;
-    const size_t begin = (size_t) wave * seg < len ? (size_t) wave * seg : len;
-    const size_t end = begin + seg < len ? begin + seg : len;
-    uint32_t total = 0;
-    for (size_t i = begin + lane; i < end; i += 64) total += in[i];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) total += __shfl_xor(total, off);
-    if (lane == 0) s_wave[wave] = total;
-    __syncthreads();
+    const int lane = threadIdx.x;
+    const uint32_t* row = hist + (size_t) blockIdx.x * n_tiles;
+    uint32_t* out = bases + (size_t) blockIdx.x * n_tiles;
     uint32_t carry = 0;
-    for (int w = 0; w < wave; ++w) carry += s_wave[w];
 #pragma unroll 4
-    for (size_t base = begin; base < end; base += 64) {
-        const size_t i = base + lane;
-        const uint32_t v = i < end ? in[i] : 0u;
+    for (uint32_t base = 0; base < n_tiles; base += 64) {
+        const uint32_t i = base + lane;
+        const uint32_t v = i < n_tiles ? row[i] : 0u;
         uint32_t incl = v;
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) {
             const uint32_t t = __shfl_up(incl, off);
             if (lane >= off) incl += t;
         }
-        if (i < end) out[i] = carry + incl - v;
+        if (i < n_tiles) out[i] = carry + incl - v;
         carry += __shfl(incl, 63);
     }
+    if (lane == 0) totals[blockIdx.x] = carry;
 }
 
 // Segment boundaries of the sorted assignment keys: offsets[c] = first position whose key is >= c
@@ -72,8 +67,8 @@ __global__ __launch_bounds__(256) void segment_bounds_kernel(
     for (uint32_t c = first; c <= key; ++c) offsets[c] = (uint32_t) i;
 }
 
-// Pass 1 of a radix step: digit histogram of one tile, stored digit-major so that one exclusive
-// scan over [digit][tile] yields the global base of every (digit, tile) pair.
+// First step of a radix pass: digit histogram of one tile, stored digit-major ([digit][tile]) so that every digit's
+// counts over the tiles are one contiguous row for digit_rows_scan_kernel.
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
     const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t n_tiles, uint32_t* __restrict__ hist
 ) {
@@ -89,18 +84,34 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
     hist[(size_t) threadIdx.x * n_tiles + blockIdx.x] = s_hist[threadIdx.x];
 }
 
-// Pass 2: stable scatter.  The tile is consumed in rounds of 256 consecutive elements; inside a
+// Third step: stable scatter.  The tile is consumed in rounds of 256 consecutive elements; inside a
 // round the rank of an element among equal digits is (equal digits in earlier wavefronts) +
 // (equal digits in lower lanes of its wavefront), the latter from eight ballots.
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift,
-    uint32_t n_tiles, const uint32_t* __restrict__ bases, uint32_t* __restrict__ keys_out,
-    uint32_t* __restrict__ vals_out, int vals_are_iota
+    uint32_t n_tiles, const uint32_t* __restrict__ bases, const uint32_t* __restrict__ totals,
+    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int vals_are_iota
 ) {
+    static_assert(SORT_THREADS == RADIX, "thread t owns digit t");
     __shared__ uint32_t s_base[RADIX];
     __shared__ uint32_t s_wave_cnt[SORT_THREADS / 64][RADIX];
+    __shared__ uint32_t s_wave_total[SORT_THREADS / 64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    s_base[tid] = bases[(size_t) tid * n_tiles + blockIdx.x];
+    {
+        // exclusive prefix of the digit totals: 64 digits per wavefront with shuffles, the four partial totals through LDS
+        const uint32_t total = totals[tid];
+        uint32_t incl = total;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const uint32_t t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) s_wave_total[wave] = incl;
+        __syncthreads();
+        uint32_t below = incl - total;
+        for (int w = 0; w < wave; ++w) below += s_wave_total[w];
+        s_base[tid] = below + bases[(size_t) tid * n_tiles + blockIdx.x];
+    }
     const size_t t0 = (size_t) blockIdx.x * SORT_TILE;
     for (int r = 0; r < SORT_TILE / SORT_THREADS; ++r) {
         const size_t i = t0 + (size_t) r * SORT_THREADS + tid;
@@ -196,7 +207,8 @@ __global__ __launch_bounds__(64) void segment_sum_deep_kernel(
             // an address built from integers is "flat" unless it says that it is global memory; flat loads would
             // make every wait a wait for all loads
             typedef const vec_t __attribute__((address_space(1))) * global_row_t;
-            return reinterpret_cast<global_row_t>(((uint64_t) hi << 32) | lo)[t_load];
+            // every row is read once per update: a non-temporal load keeps it from displacing what the caches hold
+            return __builtin_nontemporal_load(reinterpret_cast<global_row_t>(((uint64_t) hi << 32) | lo) + t_load);
         };
         vec_t ring[ROWS];
         uint64_t addresses = address_of(batch_ids(j0));
@@ -365,7 +377,7 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     // Scratch: keys/vals double buffers (4n u32), offsets (k+1), per-tile histograms.
     const uint32_t n_tiles = (uint32_t) ((n + SORT_TILE - 1) / SORT_TILE);
     const size_t hist_len = (size_t) RADIX * std::max<uint32_t>(n_tiles, 1);
-    const size_t words = 4 * n + (k + 1) + 2 * hist_len + 64;
+    const size_t words = 4 * n + (k + 1) + 2 * hist_len + RADIX + 64;
     void* ws = nullptr;
     SKM_TRY(workspace(ctx, 1, words * sizeof(uint32_t), &ws));
     uint32_t* keys_a = (uint32_t*) ws;
@@ -375,6 +387,7 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     uint32_t* offsets = vals_b + n;
     uint32_t* hist = offsets + (k + 1);
     uint32_t* bases = hist + hist_len;
+    uint32_t* totals = bases + hist_len;
 
     const uint32_t* sorted_ids = nullptr;
     if (n > 0) {
@@ -384,21 +397,29 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         const uint32_t* kin = d_idx;
         const uint32_t* vin = nullptr;
         uint32_t* kout = keys_a;
-        uint32_t* vout = vals_a;
+        // the last pass writes the ids into the context's own buffer: the pruned search of the next iteration visits
+        // the points in this order
+        void* ws_order = nullptr;
+        SKM_TRY(workspace(ctx, 4, n * sizeof(uint32_t), &ws_order));
+        ctx->cluster_order = nullptr;
+        ctx->cluster_order_n = 0;
+        uint32_t* vout = passes == 1 ? (uint32_t*) ws_order : vals_a;
         for (int p = 0; p < passes; ++p) {
             const int shift = 8 * p;
             hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, n_tiles, hist);
             SKM_HIP_TRY(hipGetLastError());
-            hipLaunchKernelGGL(exclusive_scan_kernel, dim3(1), dim3(1024), 0, ctx->stream, hist, bases, hist_len);
+            hipLaunchKernelGGL(digit_rows_scan_kernel, dim3(RADIX), dim3(64), 0, ctx->stream, hist, n_tiles, bases, totals);
             SKM_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift,
-                               n_tiles, bases, kout, vout, p == 0 ? 1 : 0);
+                               n_tiles, bases, totals, kout, vout, p == 0 ? 1 : 0);
             SKM_HIP_TRY(hipGetLastError());
             kin = kout;
             vin = vout;
             kout = (kout == keys_a) ? keys_b : keys_a;
-            vout = (vout == vals_a) ? vals_b : vals_a;
+            vout = (p + 2 == passes) ? (uint32_t*) ws_order : ((vout == vals_a) ? vals_b : vals_a);
         }
+        ctx->cluster_order = (const uint32_t*) ws_order;
+        ctx->cluster_order_n = n;
         sorted_ids = vin;
         // Sizes and segment offsets come from the sorted keys: no counting pass over the assignments.
         hipLaunchKernelGGL(segment_bounds_kernel, dim3((unsigned) ((n + 1 + 255) / 256)), dim3(256), 0, ctx->stream, kin, n,
@@ -406,6 +427,8 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         SKM_HIP_TRY(hipGetLastError());
     } else {
         sorted_ids = vals_a;
+        ctx->cluster_order = nullptr;
+        ctx->cluster_order_n = 0;
         SKM_TRY(skm_fill_u32(ctx, offsets, 0u, k + 1));
     }
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&

@@ -99,13 +99,17 @@ int device_release(int device, void* ptr) {
 }
 
 int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out) {
-    if (slot < 0 || slot >= 4) return set_error(SKM_ERR_INVALID, "bad workspace slot");
+    if (slot < 0 || slot >= skm_ctx::WS_SLOTS) return set_error(SKM_ERR_INVALID, "bad workspace slot");
     if (ctx->ws_bytes[slot] < bytes) {
         if (ctx->ws[slot]) {
             SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
             SKM_TRY(device_release(ctx->device, ctx->ws[slot]));
             ctx->ws[slot] = nullptr;
             ctx->ws_bytes[slot] = 0;
+            if (slot == 4) {
+                ctx->cluster_order = nullptr;
+                ctx->cluster_order_n = 0;
+            }
         }
         SKM_TRY(device_alloc(ctx->device, bytes, &ctx->ws[slot]));
         ctx->ws_bytes[slot] = bytes;
@@ -238,7 +242,7 @@ int skm_ctx_destroy(skm_ctx* ctx) {
         (void) hipEventDestroy(iv.stop);
     }
     for (auto e : ctx->event_pool) (void) hipEventDestroy(e);
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < skm_ctx::WS_SLOTS; ++i)
         if (ctx->ws[i]) (void) device_release(ctx->device, ctx->ws[i]);
     if (ctx->h_pinned) (void) hipHostFree(ctx->h_pinned);
     if (ctx->copy_stream) {

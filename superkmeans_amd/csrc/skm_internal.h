@@ -30,8 +30,15 @@ struct skm_ctx {
     size_t workspace_limit = size_t(24) << 30;
     int candidate_kernel = 0;  // skm_ctx_set_candidate_kernel
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
-    void* ws[4] = {nullptr, nullptr, nullptr, nullptr};
-    size_t ws_bytes[4] = {0, 0, 0, 0};
+    static constexpr int WS_SLOTS = 6;
+    void* ws[WS_SLOTS] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    size_t ws_bytes[WS_SLOTS] = {0, 0, 0, 0, 0, 0};
+    // Point ids grouped by assignment, as the last centroid update sorted them (workspace slot 4, valid for
+    // cluster_order_n points).  The pruned search visits the points in this order: neighbours in it share their
+    // centroid row and most of their candidate blocks, which then come from the cache of the compute die that
+    // fetched them first.  Any permutation of the points gives the same results.
+    const uint32_t* cluster_order = nullptr;
+    size_t cluster_order_n = 0;
     // Small pinned host buffer for scalar results.
     void* h_pinned = nullptr;
     size_t h_pinned_bytes = 0;
@@ -126,12 +133,13 @@ bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, in
 int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                                       const float* xnorm_p, const float* cnorm_p, const float* thr0,
                                       uint32_t* cand_count, uint2* cand, uint32_t cap);
+// `order`: null, or a permutation of the n points giving the sequence in which wavefronts take them.
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
-                         const float* ratios, int partial_d, float* best0, float* thr0);
+                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order);
 int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
-                      unsigned long long* d_stage_pairs);
+                      unsigned long long* d_stage_pairs, const uint32_t* order);
 int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
                             uint64_t* ids, uint32_t* n_over);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);

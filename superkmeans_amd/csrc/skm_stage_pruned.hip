@@ -100,6 +100,8 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     uint32_t* d_n_over = d_cand_count + cn;
     SKM_TRY(skm_fill_u32(ctx, d_n_over, 0u, 1));
 
+    // The order the last centroid update left, when it covers exactly these points and they are one chunk.
+    const uint32_t* order = (chunk >= n && ctx->cluster_order_n == n) ? ctx->cluster_order : nullptr;
     for (size_t i0 = 0; i0 < n; i0 += chunk) {
         const size_t m = std::min(chunk, n - i0);
         void* ws_cand = nullptr;
@@ -108,7 +110,7 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         {
             ScopedStage st(ctx, "search/seed");
             SKM_TRY(launch_seed_distance(ctx, xc, d_c, d_inout_idx + i0, (int) m, (int) d, d_ratios, (int) partial_d,
-                                         d_best0, d_thr0));
+                                         d_best0, d_thr0, order));
         }
         {
             ScopedStage st(ctx, "search/blas");
@@ -127,7 +129,7 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
             ScopedStage st(ctx, "search/pdx");
             SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
                                       (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
-                                      d_out_dist + i0, d_counts + i0, stage_arg));
+                                      d_out_dist + i0, d_counts + i0, stage_arg, order));
         }
     }
     // Points whose list overflowed (loose seeds, or points with no centroid nearby): one dense redo for

@@ -149,6 +149,37 @@ def test_automatic_choice_of_the_candidate_kernel_at_many_points(capi, ctx, orac
     assert len(mism) <= int(1e-4 * n)
 
 
+@pytest.mark.parametrize("n,d,k,partial_d,random_seeds", [(3001, 768, 1100, 96, False), (2050, 256, 1500, 32, True),
+                                                          (37, 128, 20, 16, False)])
+def test_visiting_order_left_by_the_update_does_not_change_results(capi, ctx, oracle, blobs, n, d, k, partial_d, random_seeds):
+    """After skm_update on a context, the pruned search of the same number of points takes them grouped by the
+    assignments that update sorted (eight contiguous ranges of that order, one per compute die).  Results must be
+    those of a context that never ran an update (plain point order), bit for bit, also when the order is stale
+    (sorted by other assignments than the ones the search starts from) and when the last group of four points is
+    incomplete or some dies get no group at all."""
+    X, C, prev = _setup(oracle, blobs, n, d, k, seed=7 * n + d)
+    g = np.random.default_rng(n)
+    if random_seeds:
+        prev = g.integers(0, k, n).astype(np.uint32)  # loose thresholds: overflowing lists take part as well
+    ratios = oracle.ratios(d, 1.5)
+    fresh = capi.Context(0)
+    try:
+        plain = _pruned(capi, fresh, oracle, X, C, prev, partial_d, ratios, accounting=True)
+    finally:
+        fresh.close()
+    for sorted_by in (prev, g.integers(0, k, n).astype(np.uint32)):
+        dX, dA = ctx.array(X), ctx.array(np.ascontiguousarray(sorted_by, dtype=np.uint32))
+        sums, sizes = ctx.empty((k, d)), ctx.empty(k, np.uint32)
+        capi.check(ctx.lib.skm_update(ctx.handle, dX.ptr, n, d, dA.ptr, k, sums.ptr, sizes.ptr))
+        for a in (dX, dA, sums, sizes):
+            a.free()
+        ordered = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=True)
+        assert np.array_equal(plain[0], ordered[0])
+        assert np.array_equal(plain[1].view(np.uint32), ordered[1].view(np.uint32))
+        assert plain[2] == ordered[2]
+        assert np.array_equal(plain[3], ordered[3])
+
+
 def test_pruned_with_unit_ratios_is_exact(capi, ctx, oracle, blobs):
     """With every ratio = 1 the bound partial <= full is safe, so the search must equal brute force."""
     n, d, k = 3000, 256, 1300
