@@ -173,6 +173,11 @@ int skm_edit_rows(skm_ctx* ctx, float* d_c, size_t d, const uint32_t* h_ops, siz
 /* SuperKMeans::ComputeCost (superkmeans.h:973-981): sum of n distances, accumulated in fp64 with a
  * fixed reduction tree. */
 int skm_wcss(skm_ctx* ctx, const float* d_dist, size_t n, double* h_out_cost);
+/* The same in two steps, for callers that have other work to queue in between: skm_wcss_begin queues the reduction
+ * (d_dist must stay unchanged until it has run), skm_wcss_end waits for the stream and returns the sum of the last
+ * skm_wcss_begin on this context.  Same reduction tree, same result as skm_wcss. */
+int skm_wcss_begin(skm_ctx* ctx, const float* d_dist, size_t n);
+int skm_wcss_end(skm_ctx* ctx, double* h_out_cost);
 /* SuperKMeans::ComputeShift (superkmeans.h:988-998): sum_c ||new_c - prev_c||^2. */
 int skm_shift(skm_ctx* ctx, const float* d_new, const float* d_prev, size_t k, size_t d,
               double* h_out_shift);

@@ -236,6 +236,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         hip::Check(skm_copy(ctx, this->horizontal_centroids.get(), final_centroids.get(), sizeof(float) * k * d));
         hip::Check(skm_pdxify(ctx, this->horizontal_centroids.get(), k, d, this->vertical_d, this->centroids.get(),
                               this->partial_horizontal_centroids.get()));
+        this->pdx_layout_stale = false;
         hip::Check(skm_copy(ctx, this->prev_centroids.get(), final_centroids.get(), sizeof(float) * k * d));
         hip::Check(skm_copy(ctx, this->d_assignments.get(), final_assignments.get(), sizeof(uint32_t) * total_samples));
         const bool refinement_exact = d < DIMENSION_THRESHOLD_FOR_PRUNING || k <= N_CLUSTERS_THRESHOLD_FOR_PRUNING;

@@ -313,6 +313,7 @@ class SuperKMeans {
         dbuf<float> d_norms_p(ctx, n_vectors), d_dist(ctx, n_vectors);
         hip::Check(skm_norms(ctx, d_rot.get(), n_vectors, d, partial_d, d_norms_p.get()));
         uint64_t not_pruned_total = 0;
+        EnsurePdxLayout(horizontal_centroids.get(), n_centroids);
         hip::Check(skm_assign_pruned(ctx, d_rot.get(), n_vectors, horizontal_centroids.get(), this->centroids.get(),
                                      partial_horizontal_centroids.get(), n_clusters, d, vertical_d, partial_d,
                                      pruner->DeviceRatios(), d_norms_p.get(), centroid_norms.get(), d_seed.get(),
@@ -484,6 +485,7 @@ class SuperKMeans {
                                        centroid_norms.get(), d_assignments.get(), distances.get()));
         } else {
             hip::Check(skm_norms(ctx, prev_centroids.get(), k, d, partial_d, centroid_norms.get()));
+            EnsurePdxLayout(prev_centroids.get(), k);
             std::vector<uint64_t> stage_pairs;
             if (collect_prune_accounting) stage_pairs.assign((d - vertical_d) / H_DIM_SIZE + 2, 0);
             hip::Check(skm_assign_pruned(ctx, data_to_cluster, n_samples_, prev_centroids.get(), centroids.get(),
@@ -493,6 +495,9 @@ class SuperKMeans {
                                          collect_prune_accounting ? stage_pairs.data() : nullptr));
             if (collect_prune_accounting) prune_accounting.push_back(std::move(stage_pairs));
         }
+        // The sum of the distances is queued here and collected in ComputeCost: by then the stream has been waited for
+        // anyway (cluster sizes), so the cost takes no wait of its own.
+        hip::Check(skm_wcss_begin(ctx, distances.get(), n_samples_));
         // Sums and counts (zero-filled by the kernel itself for empty clusters).
         hip::Check(skm_update(ctx, data_to_cluster, n_samples_, d, d_assignments.get(), k, horizontal_centroids.get(),
                               d_cluster_sizes.get()));
@@ -633,8 +638,17 @@ class SuperKMeans {
         if (config.angular) {
             hip::Check(skm_normalize_rows(ctx, horizontal_centroids.get(), k, d));
         }
-        hip::Check(skm_pdxify(ctx, horizontal_centroids.get(), k, d, vertical_d, centroids.get(),
-                              partial_horizontal_centroids.get()));
+        // The PDX copies are read by pruned searches only: they are brought up to date when one is about to run
+        // (EnsurePdxLayout), so exact-only clusterings never pay for the relayout.
+        pdx_layout_stale = true;
+    }
+
+    // PDX copy and dense leading columns of `rows` (the current centroids, wherever the last swap left them), if
+    // the last ConsolidateCentroids has not been followed by a relayout yet (reference superkmeans.h:962-967).
+    void EnsurePdxLayout(const float* rows, const size_t k) {
+        if (!pdx_layout_stale) return;
+        hip::Check(skm_pdxify(ctx, rows, k, d, vertical_d, centroids.get(), partial_horizontal_centroids.get()));
+        pdx_layout_stale = false;
     }
 
     // WCSS of this iteration's assignments; accumulated in fp64 on the device (superkmeans.h:973-981
@@ -642,7 +656,8 @@ class SuperKMeans {
     void ComputeCost(const size_t n_samples_) {
         prev_cost = cost;
         double c = 0.0;
-        hip::Check(skm_wcss(ctx, distances.get(), n_samples_, &c));
+        (void) n_samples_;
+        hip::Check(skm_wcss_end(ctx, &c));
         cost_f64 = c;
         cost = static_cast<float>(c);
     }
@@ -734,7 +749,7 @@ class SuperKMeans {
     /**
      * Forgy initialisation (reference superkmeans.h:1100-1142): shuffle [0, n_points) with
      * mt19937(seed) and take the first k rows of `data`; the rows land in horizontal_centroids
-     * (raw) and their rotated, PDX-laid-out copy in `centroids`.
+     * (raw) and, when no iteration will replace it, their rotated, PDX-laid-out copy in `centroids`.
      */
     void GenerateCentroids(const vector_value_t* data, const size_t n_points, const size_t k, const bool rotate,
                            const bool on_device) {
@@ -756,10 +771,15 @@ class SuperKMeans {
             GatherHostRows(staged.data(), data, indices.data(), k);
             horizontal_centroids.Upload(staged.data(), k * d);
         }
-        dbuf<float> rotated(ctx, k * d);
-        RotateOrCopy(horizontal_centroids.get(), rotated.get(), k, rotate);
-        hip::Check(skm_pdxify(ctx, rotated.get(), k, d, vertical_d, centroids.get(), nullptr));
-        hip::Check(skm_sync(ctx));
+        // The PDX copy of the initial centroids is read only if no iteration follows: the first iteration is always
+        // exact and ConsolidateCentroids replaces the copy before any pruned search.
+        pdx_layout_stale = false;
+        if (config.iters == 0) {
+            dbuf<float> rotated(ctx, k * d);
+            RotateOrCopy(horizontal_centroids.get(), rotated.get(), k, rotate);
+            hip::Check(skm_pdxify(ctx, rotated.get(), k, d, vertical_d, centroids.get(), nullptr));
+            hip::Check(skm_sync(ctx));
+        }
     }
 
     void RotateOrCopy(const float* d_in, float* d_out, const size_t n_vectors, const bool rotate) {
@@ -958,6 +978,7 @@ class SuperKMeans {
 
     bool trained = false;
     bool first_search_done = false;  // Train's first exact search ran during the upload of the rows
+    bool pdx_layout_stale = false;   // ConsolidateCentroids ran since the PDX copies were last written
     size_t n_split = 0;
     uint32_t vertical_d = 0;
     float prev_cost = 0.0f;

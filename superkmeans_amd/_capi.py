@@ -57,6 +57,8 @@ _PROTOTYPES = {
     "skm_normalize_rows": (c_int, [c_void_p, _F, c_size_t, c_size_t]),
     "skm_edit_rows": (c_int, [c_void_p, _F, c_size_t, c_void_p, c_size_t]),
     "skm_wcss": (c_int, [c_void_p, _F, c_size_t, POINTER(c_double)]),
+    "skm_wcss_begin": (c_int, [c_void_p, _F, c_size_t]),
+    "skm_wcss_end": (c_int, [c_void_p, POINTER(c_double)]),
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),

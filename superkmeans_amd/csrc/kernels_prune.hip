@@ -22,6 +22,7 @@ namespace skm {
 
 constexpr int PRUNE_WAVES = 4;
 constexpr int PRUNE_CAP = SKM_Y_BATCH_SIZE;
+constexpr int LIST_PAD = 32;  // survivors per pass of the list walk
 
 struct PruneArgs {
     const float* partial;  // n_chunk x ld_partial partial distances over the first partial_d dims
@@ -112,8 +113,8 @@ __device__ __forceinline__ int compact_survivors(uint16_t* pos, float* acc, int 
 
 template <bool VEC>
 __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
-    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
-    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
+    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];  // padded as in prune_list_kernel
+    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int p = blockIdx.x * PRUNE_WAVES + wave;
@@ -195,31 +196,35 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             // This block's slice of the point was requested one block ago; the next one is requested now.
             const float4 xv = xv_next;
             if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
-            // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.
+            // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.  Slots past
+            // the last survivor read the pad (position 0) and their sums land in the pad.
+            if (lane < LIST_PAD) pos[cnt + lane] = 0;
+            const char* blk_bytes = reinterpret_cast<const char*>(blk);
+            const uint32_t lane_bytes = (uint32_t) sub * 16u;
             for (int s0 = 0; s0 < cnt; s0 += 32) {
                 float4 cv[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
-                    const int s = s0 + 4 * u + grp;
-                    const int cpos = s < cnt ? pos[s] : pos[0];
-                    const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                    const uint32_t cpos = pos[s0 + 4 * u + grp];
+                    const float* cb = reinterpret_cast<const float*>(blk_bytes + ((cpos << 8) | lane_bytes));
                     if (VEC) {
                         cv[u] = *reinterpret_cast<const float4*>(cb);
                     } else {
                         cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
                     }
                 }
+                float mine = 0.0f;
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
-                    const int s = s0 + 4 * u + grp;
                     float e, part = 0.0f;
                     e = xv.x - cv[u].x; part += e * e;
                     e = xv.y - cv[u].y; part += e * e;
                     e = xv.z - cv[u].z; part += e * e;
                     e = xv.w - cv[u].w; part += e * e;
                     part = group16_sum(part);
-                    if (s < cnt && sub == 0) acc[s] += part;
+                    mine = sub == u ? part : mine;
                 }
+                if (sub < 8) acc[s0 + 4 * sub + grp] += mine;
             }
             dims_seen += SKM_H_DIM_SIZE;
             thr = best * a.ratios[dims_seen];
@@ -380,8 +385,11 @@ struct PruneListArgs {
 
 template <bool VEC, bool ACCT>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
 __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneListArgs a) {
-    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP];
-    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP];
+    // LIST_PAD slots past the live survivors: a pass of 32 gathers reads positions and adds partial sums without
+    // asking whether a slot is live; the pad positions are kept at 0 (a valid centroid of any batch), what is added to
+    // the pad sums is never read.
+    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];
+    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];
     __shared__ float s_parts[PRUNE_WAVES][16 * 8];  // [block of the group][survivor]
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -413,7 +421,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     if (lane < n_cand) entry = list[lane];
 
     while (cur < n_cand) {
-        const uint32_t jb = (uint32_t) __shfl((int) entry.x, (int) (cur - chunk0)) / SKM_Y_BATCH_SIZE;
+        // the same value in every lane: saying so keeps the batch's base pointers in scalar registers
+        const uint32_t jb = (uint32_t) __builtin_amdgcn_readfirstlane(__shfl((int) entry.x, (int) (cur - chunk0))) / SKM_Y_BATCH_SIZE;
         const int base = (int) jb * SKM_Y_BATCH_SIZE;
         const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
         const uint32_t prev_top_1 = best_idx;
@@ -507,31 +516,37 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
             } else {
                 if (ACCT && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
                 const float4 xv = load_x4<VEC>(xq + V + hb * SKM_H_DIM_SIZE + sub * 4);
-                // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.
+                // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.  Slots past
+                // the last survivor read the pad (position 0) and their sums land in the pad.
+                if (lane < LIST_PAD) pos[cnt + lane] = 0;
+                const char* blk_bytes = reinterpret_cast<const char*>(blk);
+                const uint32_t lane_bytes = (uint32_t) sub * 16u;
                 for (int s0 = 0; s0 < cnt; s0 += 32) {
                     float4 cv[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
-                        const int s = s0 + 4 * u + grp;
-                        const int cpos = s < cnt ? pos[s] : pos[0];
-                        const float* cb = blk + (int64_t) cpos * SKM_H_DIM_SIZE + sub * 4;
+                        const uint32_t cpos = pos[s0 + 4 * u + grp];
+                        const float* cb = reinterpret_cast<const float*>(blk_bytes + ((cpos << 8) | lane_bytes));
                         if (VEC) {
                             cv[u] = *reinterpret_cast<const float4*>(cb);
                         } else {
                             cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
                         }
                     }
+                    // all 16 lanes of a group hold the sum of each of its eight survivors: lane u of the group keeps
+                    // the u-th and the first eight lanes add theirs in one go
+                    float mine = 0.0f;
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
-                        const int s = s0 + 4 * u + grp;
                         float e, part = 0.0f;
                         e = xv.x - cv[u].x; part += e * e;
                         e = xv.y - cv[u].y; part += e * e;
                         e = xv.z - cv[u].z; part += e * e;
                         e = xv.w - cv[u].w; part += e * e;
                         part = group16_sum(part);
-                        if (s < cnt && sub == 0) acc[s] += part;
+                        mine = sub == u ? part : mine;
                     }
+                    if (sub < 8) acc[s0 + 4 * sub + grp] += mine;
                 }
                 hb += 1;
                 dims_seen += SKM_H_DIM_SIZE;

@@ -16,9 +16,12 @@
 namespace skm {
 
 constexpr int SORT_THREADS = 256;
-// Elements per workgroup and pass.  Smaller tiles give more workgroups but shorter runs of equal digits per tile: at
-// 1,024 the scatter of a pass over random low digits writes 16-byte runs and takes longer than at 4,096.
-constexpr int SORT_TILE = 4096;
+// Elements per workgroup and pass.  Smaller tiles give more workgroups but shorter runs of equal digits per tile: with a
+// million keys the scatter of a pass over random low digits writes 16-byte runs at 1,024 and takes longer than at
+// 4,096.  A sort of a few ten thousand keys (a fine clustering) is a matter of latency instead: ten workgroups of
+// sixteen rounds each, so there the small tile is the faster one.
+constexpr int SORT_TILE = 4096, SORT_TILE_FEW_KEYS = 1024;
+constexpr size_t SORT_FEW_KEYS = size_t(1) << 18;
 constexpr int RADIX = 256;
 
 // Second step of a radix pass.  The histograms are stored digit-major, so the global base of a (digit, tile) pair is
@@ -70,13 +73,13 @@ __global__ __launch_bounds__(256) void segment_bounds_kernel(
 // First step of a radix pass: digit histogram of one tile, stored digit-major ([digit][tile]) so that every digit's
 // counts over the tiles are one contiguous row for digit_rows_scan_kernel.
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
-    const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t n_tiles, uint32_t* __restrict__ hist
+    const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t n_tiles, int tile, uint32_t* __restrict__ hist
 ) {
     __shared__ uint32_t s_hist[RADIX];
     s_hist[threadIdx.x] = 0;
     __syncthreads();
-    const size_t t0 = (size_t) blockIdx.x * SORT_TILE;
-    for (int r = 0; r < SORT_TILE / SORT_THREADS; ++r) {
+    const size_t t0 = (size_t) blockIdx.x * tile;
+    for (int r = 0; r < tile / SORT_THREADS; ++r) {
         const size_t i = t0 + (size_t) r * SORT_THREADS + threadIdx.x;
         if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & (RADIX - 1)], 1u);
     }
@@ -89,7 +92,7 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
 // (equal digits in lower lanes of its wavefront), the latter from eight ballots.
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift,
-    uint32_t n_tiles, const uint32_t* __restrict__ bases, const uint32_t* __restrict__ totals,
+    uint32_t n_tiles, int tile, const uint32_t* __restrict__ bases, const uint32_t* __restrict__ totals,
     uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int vals_are_iota
 ) {
     static_assert(SORT_THREADS == RADIX, "thread t owns digit t");
@@ -112,8 +115,8 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         for (int w = 0; w < wave; ++w) below += s_wave_total[w];
         s_base[tid] = below + bases[(size_t) tid * n_tiles + blockIdx.x];
     }
-    const size_t t0 = (size_t) blockIdx.x * SORT_TILE;
-    for (int r = 0; r < SORT_TILE / SORT_THREADS; ++r) {
+    const size_t t0 = (size_t) blockIdx.x * tile;
+    for (int r = 0; r < tile / SORT_THREADS; ++r) {
         const size_t i = t0 + (size_t) r * SORT_THREADS + tid;
         const bool in = i < n;
 #pragma unroll
@@ -334,11 +337,23 @@ __global__ __launch_bounds__(256) void reduce_stage2_kernel(const double* __rest
     if (threadIdx.x == 0) out[0] = s[0];
 }
 
-static int reduce_to_host(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_out) {
+// Result slots in the context's pinned host buffer (8 bytes each).  The second reduction stage writes its result
+// straight into the slot, which the device reaches through the buffer's host address: no copy operation, the host reads
+// the slot after its next wait on the stream.
+enum { SLOT_SCALAR = 0, SLOT_OVERFLOW = 1, SLOT_NOT_PRUNED = 2, SLOT_WCSS = 3, N_RESULT_SLOTS = 8 };
+
+static int result_slot(skm_ctx* ctx, int slot, double** out) {
+    void* hp = nullptr;
+    SKM_TRY(pinned(ctx, N_RESULT_SLOTS * sizeof(double), &hp));
+    *out = (double*) hp + slot;
+    return SKM_OK;
+}
+
+// Queues the reduction; the result is in *h_slot once the stream has been waited for.
+static int reduce_enqueue(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_slot) {
     void* ws = nullptr;
     SKM_TRY(workspace(ctx, 3, (REDUCE_BLOCKS + 8) * sizeof(double), &ws));
     double* partial = (double*) ws;
-    double* result = partial + REDUCE_BLOCKS;
     if (mode == 0)
         hipLaunchKernelGGL(reduce_stage1_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
     else if (mode == 1)
@@ -346,18 +361,33 @@ static int reduce_to_host(skm_ctx* ctx, int mode, const float* a, const float* b
     else
         hipLaunchKernelGGL(reduce_stage1_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
     SKM_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(reduce_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, result);
-    SKM_HIP_TRY(hipGetLastError());
-    void* hp = nullptr;
-    SKM_TRY(pinned(ctx, 64, &hp));
-    SKM_HIP_TRY(hipMemcpyAsync(hp, result, sizeof(double), hipMemcpyDeviceToHost, ctx->stream));
+    hipLaunchKernelGGL(reduce_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, h_slot);
+    return check_hip(hipGetLastError(), "reduce_stage2_kernel launch");
+}
+
+static int reduce_to_host(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_out) {
+    double* slot = nullptr;
+    SKM_TRY(result_slot(ctx, SLOT_SCALAR, &slot));
+    SKM_TRY(reduce_enqueue(ctx, mode, a, b, n, slot));
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-    *h_out = *(double*) hp;
+    *h_out = *(volatile double*) slot;
     return SKM_OK;
 }
 
 int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_out) {
     return reduce_to_host(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, h_out);
+}
+
+int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot) {
+    SKM_TRY(result_slot(ctx, SLOT_NOT_PRUNED, h_slot));
+    return reduce_enqueue(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, *h_slot);
+}
+
+int overflow_count_slot(skm_ctx* ctx, uint32_t** h_slot) {
+    double* slot = nullptr;
+    SKM_TRY(result_slot(ctx, SLOT_OVERFLOW, &slot));
+    *h_slot = reinterpret_cast<uint32_t*>(slot);
+    return SKM_OK;
 }
 
 } // namespace skm
@@ -375,7 +405,8 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
     SKM_REQUIRE(n == 0 || (d_x && d_idx), "null input");
     ScopedStage st(ctx, "update_centroids");
     // Scratch: keys/vals double buffers (4n u32), offsets (k+1), per-tile histograms.
-    const uint32_t n_tiles = (uint32_t) ((n + SORT_TILE - 1) / SORT_TILE);
+    const int tile = n <= SORT_FEW_KEYS ? SORT_TILE_FEW_KEYS : SORT_TILE;
+    const uint32_t n_tiles = (uint32_t) ((n + tile - 1) / tile);
     const size_t hist_len = (size_t) RADIX * std::max<uint32_t>(n_tiles, 1);
     const size_t words = 4 * n + (k + 1) + 2 * hist_len + RADIX + 64;
     void* ws = nullptr;
@@ -406,12 +437,12 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         uint32_t* vout = passes == 1 ? (uint32_t*) ws_order : vals_a;
         for (int p = 0; p < passes; ++p) {
             const int shift = 8 * p;
-            hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, n_tiles, hist);
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, n_tiles, tile, hist);
             SKM_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL(digit_rows_scan_kernel, dim3(RADIX), dim3(64), 0, ctx->stream, hist, n_tiles, bases, totals);
             SKM_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift,
-                               n_tiles, bases, totals, kout, vout, p == 0 ? 1 : 0);
+                               n_tiles, tile, bases, totals, kout, vout, p == 0 ? 1 : 0);
             SKM_HIP_TRY(hipGetLastError());
             kin = kout;
             vin = vout;
@@ -525,6 +556,24 @@ int skm_wcss(skm_ctx* ctx, const float* d_dist, size_t n, double* h_out_cost) {
     SKM_REQUIRE(n == 0 || d_dist, "null input");
     ScopedStage st(ctx, "compute_cost");
     return reduce_to_host(ctx, 0, d_dist, nullptr, n, h_out_cost);
+}
+
+int skm_wcss_begin(skm_ctx* ctx, const float* d_dist, size_t n) {
+    SKM_REQUIRE(ctx, "null argument");
+    SKM_REQUIRE(n == 0 || d_dist, "null input");
+    ScopedStage st(ctx, "compute_cost");
+    double* slot = nullptr;
+    SKM_TRY(result_slot(ctx, SLOT_WCSS, &slot));
+    return reduce_enqueue(ctx, 0, d_dist, nullptr, n, slot);
+}
+
+int skm_wcss_end(skm_ctx* ctx, double* h_out_cost) {
+    SKM_REQUIRE(ctx && h_out_cost, "null argument");
+    double* slot = nullptr;
+    SKM_TRY(result_slot(ctx, SLOT_WCSS, &slot));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    *h_out_cost = *(volatile double*) slot;
+    return SKM_OK;
 }
 
 int skm_shift(skm_ctx* ctx, const float* d_new, const float* d_prev, size_t k, size_t d, double* h_out_shift) {

@@ -17,6 +17,8 @@
 
 namespace skm {
 int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_out);
+int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot);
+int overflow_count_slot(skm_ctx* ctx, uint32_t** h_slot);
 }
 
 using namespace skm;
@@ -133,12 +135,16 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         }
     }
     // Points whose list overflowed (loose seeds, or points with no centroid nearby): one dense redo for
-    // all of them: gather, dense partial distances + dense pruning, scatter the results back.
-    void* h_pin = nullptr;
-    SKM_TRY(pinned(ctx, 64, &h_pin));
-    SKM_HIP_TRY(hipMemcpyAsync(h_pin, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    // all of them: gather, dense partial distances + dense pruning, scatter the results back.  The sum of the
+    // per-point counts is queued before the number of overflowing points is known and both arrive with one wait;
+    // it is taken again only if a redo changed some counts.
+    double* h_not_pruned = nullptr;
+    if (h_out_not_pruned) SKM_TRY(reduce_u32_sum_enqueue(ctx, d_counts, n, &h_not_pruned));
+    uint32_t* h_n_over = nullptr;
+    SKM_TRY(overflow_count_slot(ctx, &h_n_over));
+    SKM_HIP_TRY(hipMemcpyAsync(h_n_over, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-    const size_t mo = *(volatile uint32_t*) h_pin;
+    const size_t mo = *(volatile uint32_t*) h_n_over;
     if (mo > 0) {
         ScopedStage st(ctx, "search/overflow");
         void* ws_o = nullptr;
@@ -157,8 +163,8 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_over_ids, (int) mo, d_counts));
     }
     if (h_out_not_pruned) {
-        double total = 0.0;
-        SKM_TRY(reduce_u32_sum_to_host(ctx, d_counts, n, &total));
+        double total = *(volatile double*) h_not_pruned;
+        if (mo > 0) SKM_TRY(reduce_u32_sum_to_host(ctx, d_counts, n, &total));
         *h_out_not_pruned = (uint64_t) total;
     }
     if (h_out_stage_pairs) {

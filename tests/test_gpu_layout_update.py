@@ -91,7 +91,18 @@ def test_wcss_and_shift(capi, ctx):
     assert abs(out.value - exact) <= 1e-6 * exact
     capi.check(ctx.lib.skm_wcss(ctx.handle, dd.ptr, 0, ctypes.byref(out)))
     assert out.value == 0.0
-    for arr in (dd, da, db):
+    # the two-step form: other reductions and an update run between the two calls and leave the pending sum alone
+    capi.check(ctx.lib.skm_wcss(ctx.handle, dd.ptr, dist.size, ctypes.byref(out)))
+    whole = out.value
+    capi.check(ctx.lib.skm_wcss_begin(ctx.handle, dd.ptr, dist.size))
+    capi.check(ctx.lib.skm_shift(ctx.handle, da.ptr, db.ptr, 777, 130, ctypes.byref(out)))
+    assign = ctx.array((np.arange(777) % 10).astype(np.uint32))
+    sums, sizes = ctx.empty((10, 130)), ctx.empty(10, np.uint32)
+    capi.check(ctx.lib.skm_update(ctx.handle, da.ptr, 777, 130, assign.ptr, 10, sums.ptr, sizes.ptr))
+    capi.check(ctx.lib.skm_wcss(ctx.handle, da.ptr, 777 * 130, ctypes.byref(out)))
+    capi.check(ctx.lib.skm_wcss_end(ctx.handle, ctypes.byref(out)))
+    assert out.value == whole
+    for arr in (dd, da, db, assign, sums, sizes):
         arr.free()
 
 
