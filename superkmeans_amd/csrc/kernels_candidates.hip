@@ -334,8 +334,9 @@ bool gemm_candidates_stationary_serves(const float* C, int k, const float* X, in
     if ((int64_t) groups * 8 > ld) return false;
     // centroid rows are addressed with 32-bit byte offsets, the tiles requested past the end included
     if (((int64_t) k + 4 * CS_TN) * ld * 4 >= (int64_t(1) << 32)) return false;
-    // a workgroup owns 256 points: below a few rounds of workgroups the 128-point kernel fills the chip better
-    return whatever_n || n >= 512 * CS_POINTS;
+    // a workgroup owns 256 points: with fewer workgroups than about three quarters of the compute units the 128-point
+    // kernel fills the chip better (measured at k = 1,000: 20 % faster than that kernel at 100,000 points, 8 % at 50,000)
+    return whatever_n || n >= 192 * CS_POINTS;
 }
 
 int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,

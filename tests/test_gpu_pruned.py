@@ -133,8 +133,8 @@ def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs)
 
 
 def test_automatic_choice_of_the_candidate_kernel_at_many_points(capi, ctx, oracle, blobs):
-    """131,072 points and more select the register-stationary kernel by themselves; checked against the oracle."""
-    n, d, k, partial_d = 140000, 128, 1100, 32
+    """49,152 points and more select the register-stationary kernel by themselves; checked against the oracle."""
+    n, d, k, partial_d = 60000, 128, 1100, 32
     X, C, prev = _setup(oracle, blobs, n, d, k, seed=9)
     ratios = oracle.ratios(d, 1.5)
     auto = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios)
