@@ -38,16 +38,18 @@ PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBPS = 8000.0
 
 
-# L2 <-> fabric bytes of one exact search (the two gemm_argmin_kernel launches of an Assign pass), from two rocprofv3 --pmc passes (FETCH_SIZE, then
-# WRITE_SIZE, KiB per dispatch) scaled by what the same counters read for a copy kernel of known size
-# (FETCH_SIZE x 1.943, WRITE_SIZE x 1.000); counters cannot be read from inside this process, so the figure is
-# kept per workload shape (n, d, k) and is null for shapes that were not profiled.
+# Counter figures cannot be read from inside this process: they are recorded here from the rocprofv3 --pmc runs whose
+# summaries are under profiles/ (FETCH_SIZE and WRITE_SIZE in KiB per dispatch, scaled by what the same counters read for a
+# copy kernel of known size: FETCH_SIZE x 1.943, WRITE_SIZE x 1.000), per workload shape, and are null for shapes that were
+# not profiled.  They describe the build the summaries were taken with; a change to a kernel needs a new profile run.
+#   profiles/gemm_argmin_kernel_assign_n1M_d1024_k10k_hbm_traffic.md: the two gemm_argmin_kernel launches of an Assign pass
 MEASURED_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000): int(((31_523_194 + 2_005_616) * 1.943 + 609_375 + 7_812) * 1024),
+    (1_000_000, 1024, 10_000): int(((31_470_719 + 2_006_672) * 1.943 + 609_375 + 7_812) * 1024),
 }
-# The same counters summed over the seed, list-walk and overflow kernels of one Train of (n, d, k, iterations); recorded
-# from the profile named in profiles/ for that shape, null where none was taken.
-MEASURED_PRUNE_TRAFFIC_BYTES = {}
+#   same file: every seed_distance_kernel, prune_list_kernel and prune_kernel launch of one Train of (n, d, k, iterations)
+MEASURED_PRUNE_TRAFFIC_BYTES = {
+    (1_000_000, 1024, 10_000, 10): int((50_265_137 * 1.943 + 1_471_834) * 1024),
+}
 
 
 # name -> (n, d, k, Train iterations, hierarchical, description of the generator)
@@ -218,10 +220,13 @@ def main():
             if blocks_visited > 0:
                 stage["prune"]["pair_blocks_visited"] = blocks_visited
                 stage["prune"]["ns_per_pair_block"] = round(stage["prune"]["ms"] * 1e6 / blocks_visited, 4)
+            # `achieved` counts every gathered 256-byte centroid block as traffic (most are served by L2); the bytes that
+            # actually leave the L2s, from the counters, and the fraction of the HBM figure they amount to
             measured = MEASURED_PRUNE_TRAFFIC_BYTES.get((n, d, k, len(stats)))
-            if measured:
-                stage["prune"]["measured_bytes"] = measured
-                stage["prune"]["measured_frac"] = round(measured / (stage["prune"]["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4)
+            stage["prune"]["measured_bytes"] = measured
+            stage["prune"]["measured_frac"] = round(measured / (stage["prune"]["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4) \
+                if measured else None
+            stage["prune"]["bound_note"] = "instruction issue and L2 gathers, not HBM: see ns_per_pair_block"
         if hierarchical:
             train["phases"] = {name: {"iterations": len(v), "final_objective": (v[-1].objective if v and name != "fineclustering" else None)}
                                for name, v in phase_stats.items()}

@@ -117,8 +117,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
     __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int p = blockIdx.x * PRUNE_WAVES + wave;
-    if (p >= a.n) return;
+    const int p = point_of_wave(nullptr, a.n, PRUNE_WAVES);  // consecutive rows stay on one compute die
+    if (p < 0) return;
     uint16_t* pos = s_pos[wave];
     float* acc = s_acc[wave];
     const int d = a.d, V = a.vertical_d, dp = a.partial_d;
@@ -623,12 +623,25 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
 }
 
 // Appends the ids (id_offset + chunk-local index) of the points whose candidate list overflowed.
+// With a visiting order the points are examined in that order, so that neighbours in the list of overflowing points
+// tend to be neighbours in the order (the list is only as ordered as the atomics of concurrently running wavefronts
+// leave it; its order changes where the dense redo finds its centroid blocks, not what it computes).
 __global__ __launch_bounds__(256) void collect_overflow_kernel(
     const uint32_t* __restrict__ cand_count, int n, uint32_t cap, uint64_t id_offset, uint64_t* __restrict__ ids,
-    uint32_t* __restrict__ n_over
+    uint32_t* __restrict__ n_over, const uint32_t* __restrict__ order
 ) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n && cand_count[i] > cap) ids[atomicAdd(n_over, 1u)] = id_offset + (uint64_t) i;
+    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+    if (slot >= n) return;
+    const uint32_t i = order ? order[slot] : (uint32_t) slot;
+    const bool over = cand_count[i] > cap;
+    // one atomic per wavefront: its overflowing points take consecutive entries in lane order
+    const unsigned long long mask = __ballot(over);
+    if (mask == 0) return;
+    const int lane = threadIdx.x & 63;
+    uint32_t base = 0;
+    if (lane == __ffsll((long long) mask) - 1) base = atomicAdd(n_over, (uint32_t) __popcll(mask));
+    base = (uint32_t) __shfl((int) base, __ffsll((long long) mask) - 1);
+    if (over) ids[base + (uint32_t) __popcll(mask & ((1ull << lane) - 1ull))] = id_offset + (uint64_t) i;
 }
 
 __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ in, const uint64_t* __restrict__ ids, int m, uint32_t* __restrict__ out) {
@@ -677,10 +690,10 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
 }
 
 int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
-                            uint64_t* ids, uint32_t* n_over) {
+                            uint64_t* ids, uint32_t* n_over, const uint32_t* order) {
     if (n <= 0) return SKM_OK;
     hipLaunchKernelGGL(collect_overflow_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, cand_count, n, cap,
-                       id_offset, ids, n_over);
+                       id_offset, ids, n_over, order);
     return check_hip(hipGetLastError(), "collect_overflow_kernel launch");
 }
 
@@ -708,7 +721,7 @@ int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const f
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(c) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
-    dim3 grid((n_chunk + PRUNE_WAVES - 1) / PRUNE_WAVES), block(PRUNE_WAVES * 64);
+    dim3 grid(die_striped_groups(n_chunk, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (vec)
         hipLaunchKernelGGL(prune_kernel<true>, grid, block, 0, ctx->stream, a);
     else

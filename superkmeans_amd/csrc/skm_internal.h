@@ -141,7 +141,7 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order);
 int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
-                            uint64_t* ids, uint32_t* n_over);
+                            uint64_t* ids, uint32_t* n_over, const uint32_t* order);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 

@@ -54,6 +54,29 @@ int dense_block(skm_ctx* ctx, const float* d_x, size_t m, const float* d_c, cons
     return SKM_OK;
 }
 
+// Dense search of the points `d_ids` from their seeds in d_inout_idx: gather, dense partial distances + dense pruning
+// over all batches, results scattered back.
+int dense_redo(skm_ctx* ctx, int slot, const float* d_x, const uint64_t* d_ids, size_t mo, const float* d_c, const float* d_pdx,
+               const float* d_aux, size_t k, size_t d, size_t vertical_d, uint32_t partial_d, const float* d_ratios,
+               const float* d_xnorm_p, const float* d_cnorm_p, uint32_t* d_inout_idx, float* d_out_dist, uint32_t* d_counts,
+               unsigned long long* d_stage) {
+    void* ws_o = nullptr;
+    SKM_TRY(workspace(ctx, slot, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
+    float* xo = (float*) ws_o;
+    float* xnorm_o = xo + mo * d;
+    uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
+    float* dist_o = (float*) (idx_o + align_up(mo, 64));
+    uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
+    SKM_TRY(skm_gather_rows(ctx, d_x, d, d_ids, mo, xo, d_xnorm_p, xnorm_o));
+    SKM_TRY(launch_gather_u32(ctx, d_inout_idx, d_ids, (int) mo, idx_o));
+    SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p, idx_o, dist_o,
+                        cnt_o, d_stage));
+    SKM_TRY(launch_scatter_u32(ctx, idx_o, d_ids, (int) mo, d_inout_idx));
+    SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_ids, (int) mo, (uint32_t*) d_out_dist));
+    SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_ids, (int) mo, d_counts));
+    return SKM_OK;
+}
+
 } // namespace
 
 extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const float* d_c, const float* d_pdx,
@@ -126,7 +149,7 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
                 SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
                                                d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
         }
-        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over));
+        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over, order));
         {
             ScopedStage st(ctx, "search/pdx");
             SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
@@ -147,20 +170,8 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     const size_t mo = *(volatile uint32_t*) h_n_over;
     if (mo > 0) {
         ScopedStage st(ctx, "search/overflow");
-        void* ws_o = nullptr;
-        SKM_TRY(workspace(ctx, 3, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
-        float* xo = (float*) ws_o;
-        float* xnorm_o = xo + mo * d;
-        uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
-        float* dist_o = (float*) (idx_o + align_up(mo, 64));
-        uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
-        SKM_TRY(skm_gather_rows(ctx, d_x, d, d_over_ids, mo, xo, d_xnorm_p, xnorm_o));
-        SKM_TRY(launch_gather_u32(ctx, d_inout_idx, d_over_ids, (int) mo, idx_o));
-        SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p, idx_o,
-                            dist_o, cnt_o, stage_arg));
-        SKM_TRY(launch_scatter_u32(ctx, idx_o, d_over_ids, (int) mo, d_inout_idx));
-        SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_over_ids, (int) mo, (uint32_t*) d_out_dist));
-        SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_over_ids, (int) mo, d_counts));
+        SKM_TRY(dense_redo(ctx, 3, d_x, d_over_ids, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, d_xnorm_p,
+                           d_cnorm_p, d_inout_idx, d_out_dist, d_counts, stage_arg));
     }
     if (h_out_not_pruned) {
         double total = *(volatile double*) h_not_pruned;
