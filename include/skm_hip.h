@@ -163,6 +163,9 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
 /* First loop of SuperKMeans::ConsolidateCentroids (superkmeans.h:940-951): c *= float(1.0 / size)
  * for every non-empty cluster. */
 int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d);
+/* The same, and the sizes arrive in h_sizes (k entries) with the one wait on the stream the call ends with: the next
+ * step of ConsolidateCentroids, SplitClusters, decides on the host from the sizes. */
+int skm_scale_by_size_fetch(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d, uint32_t* h_sizes);
 /* SuperKMeans::PostprocessCentroids (superkmeans.h:1357-1371): c /= ||c||. */
 int skm_normalize_rows(skm_ctx* ctx, float* d_c, size_t k, size_t d);
 /* Row edits of SplitClusters (superkmeans.h:905-920; hierarchical_superkmeans.h:606-625,665-673),

@@ -632,8 +632,7 @@ class SuperKMeans {
 
     // Means, empty-cluster handling, optional normalisation, PDX relayout (superkmeans.h:936-968).
     void ConsolidateCentroids(const size_t n_samples_, const size_t k) {
-        hip::Check(skm_scale_by_size(ctx, horizontal_centroids.get(), d_cluster_sizes.get(), k, d));
-        d_cluster_sizes.Download(cluster_sizes.get(), k);
+        hip::Check(skm_scale_by_size_fetch(ctx, horizontal_centroids.get(), d_cluster_sizes.get(), k, d, cluster_sizes.get()));
         SplitClusters(n_samples_, k);
         if (config.angular) {
             hip::Check(skm_normalize_rows(ctx, horizontal_centroids.get(), k, d));

@@ -93,7 +93,8 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
     const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift,
     uint32_t n_tiles, int tile, const uint32_t* __restrict__ bases, const uint32_t* __restrict__ totals,
-    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int vals_are_iota
+    uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int vals_are_iota,
+    uint32_t* __restrict__ offsets_out, uint32_t k
 ) {
     static_assert(SORT_THREADS == RADIX, "thread t owns digit t");
     __shared__ uint32_t s_base[RADIX];
@@ -114,6 +115,12 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
         uint32_t below = incl - total;
         for (int w = 0; w < wave; ++w) below += s_wave_total[w];
         s_base[tid] = below + bases[(size_t) tid * n_tiles + blockIdx.x];
+        // A sort of one pass (k <= 256): the digit is the key, so the number of keys below digit c is where the
+        // segment of centroid c starts; offsets_out[k] is the number of keys below k.
+        if (offsets_out && blockIdx.x == 0) {
+            if ((uint32_t) tid <= k) offsets_out[tid] = below;
+            if (k == RADIX && tid == 0) offsets_out[RADIX] = (uint32_t) n;
+        }
     }
     const size_t t0 = (size_t) blockIdx.x * tile;
     for (int r = 0; r < tile / SORT_THREADS; ++r) {
@@ -243,10 +250,11 @@ __global__ __launch_bounds__(64) void segment_sum_deep_kernel(
 }
 
 __global__ __launch_bounds__(256) void scale_by_size_kernel(
-    float* __restrict__ sums, const uint32_t* __restrict__ sizes, size_t k, size_t d
+    float* __restrict__ sums, const uint32_t* __restrict__ sizes, size_t k, size_t d, uint32_t* __restrict__ sizes_copy
 ) {
     const size_t c = blockIdx.x;
     const uint32_t s = sizes[c];
+    if (sizes_copy && threadIdx.x == 0) sizes_copy[c] = s;  // pinned host memory: the host reads the sizes after its wait
     if (s == 0) return;
     const float mult = (float) (1.0 / (double) s);  // float mult_factor = 1.0 / cluster_sizes[i]
     float* row = sums + c * d;
@@ -299,13 +307,16 @@ __global__ __launch_bounds__(256) void edit_rows_kernel(float* __restrict__ c, s
 
 constexpr int REDUCE_BLOCKS = 512;
 
-// Fixed-shape two-stage reductions in fp64: block b sums elements b*256+tid, +512*256, ... so the
-// association depends only on the element count.
+// Fixed-shape two-stage reductions in fp64 in one launch: block b sums elements b*256+tid, +512*256, ... and the
+// block that finishes last (a counter tells it) adds the 512 block sums in a fixed tree, so the association depends
+// only on the element count, never on which block came last.  The counter is left at zero for the next launch.
 template <int MODE>  // 0: sum a[i]; 1: sum (a[i]-b[i])^2; 2: sum of uint32 a[i] (as exact integers)
-__global__ __launch_bounds__(256) void reduce_stage1_kernel(
-    const float* __restrict__ a, const float* __restrict__ b, size_t n, double* __restrict__ partial
+__global__ __launch_bounds__(256) void reduce_kernel(
+    const float* __restrict__ a, const float* __restrict__ b, size_t n, double* __restrict__ partial,
+    uint32_t* __restrict__ counter, double* __restrict__ out
 ) {
     __shared__ double s[256];
+    __shared__ uint32_t s_done;
     double acc = 0.0;
     for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) REDUCE_BLOCKS * 256) {
         if (MODE == 0) {
@@ -323,21 +334,28 @@ __global__ __launch_bounds__(256) void reduce_stage1_kernel(
         if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
         __syncthreads();
     }
-    if (threadIdx.x == 0) partial[blockIdx.x] = s[0];
-}
-
-__global__ __launch_bounds__(256) void reduce_stage2_kernel(const double* __restrict__ partial, double* __restrict__ out) {
-    __shared__ double s[256];
-    s[threadIdx.x] = partial[threadIdx.x] + partial[threadIdx.x + 256];
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x] = s[0];
+        __threadfence();  // the block sum is visible device-wide before the counter says so
+        s_done = atomicAdd(counter, 1u);
+    }
+    __syncthreads();
+    if (s_done != REDUCE_BLOCKS - 1) return;
+    __threadfence();
+    const volatile double* all = partial;  // written by other compute units: read past this one's cache
+    s[threadIdx.x] = all[threadIdx.x] + all[threadIdx.x + 256];
     __syncthreads();
     for (int off = 128; off > 0; off >>= 1) {
         if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
         __syncthreads();
     }
-    if (threadIdx.x == 0) out[0] = s[0];
+    if (threadIdx.x == 0) {
+        out[0] = s[0];
+        *counter = 0u;
+    }
 }
 
-// Result slots in the context's pinned host buffer (8 bytes each).  The second reduction stage writes its result
+// Result slots in the context's pinned host buffer (8 bytes each).  The reduction writes its result
 // straight into the slot, which the device reaches through the buffer's host address: no copy operation, the host reads
 // the slot after its next wait on the stream.
 enum { SLOT_SCALAR = 0, SLOT_OVERFLOW = 1, SLOT_NOT_PRUNED = 2, SLOT_WCSS = 3, N_RESULT_SLOTS = 8 };
@@ -354,15 +372,15 @@ static int reduce_enqueue(skm_ctx* ctx, int mode, const float* a, const float* b
     void* ws = nullptr;
     SKM_TRY(workspace(ctx, 3, (REDUCE_BLOCKS + 8) * sizeof(double), &ws));
     double* partial = (double*) ws;
+    uint32_t* counter = nullptr;
+    SKM_TRY(reduction_counter(ctx, &counter));
     if (mode == 0)
-        hipLaunchKernelGGL(reduce_stage1_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
+        hipLaunchKernelGGL(reduce_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
     else if (mode == 1)
-        hipLaunchKernelGGL(reduce_stage1_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
+        hipLaunchKernelGGL(reduce_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
     else
-        hipLaunchKernelGGL(reduce_stage1_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial);
-    SKM_HIP_TRY(hipGetLastError());
-    hipLaunchKernelGGL(reduce_stage2_kernel, dim3(1), dim3(256), 0, ctx->stream, partial, h_slot);
-    return check_hip(hipGetLastError(), "reduce_stage2_kernel launch");
+        hipLaunchKernelGGL(reduce_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
+    return check_hip(hipGetLastError(), "reduce_kernel launch");
 }
 
 static int reduce_to_host(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_out) {
@@ -442,7 +460,8 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
             hipLaunchKernelGGL(digit_rows_scan_kernel, dim3(RADIX), dim3(64), 0, ctx->stream, hist, n_tiles, bases, totals);
             SKM_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift,
-                               n_tiles, tile, bases, totals, kout, vout, p == 0 ? 1 : 0);
+                               n_tiles, tile, bases, totals, kout, vout, p == 0 ? 1 : 0,
+                               passes == 1 ? offsets : (uint32_t*) nullptr, (uint32_t) k);
             SKM_HIP_TRY(hipGetLastError());
             kin = kout;
             vin = vout;
@@ -452,10 +471,13 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         ctx->cluster_order = (const uint32_t*) ws_order;
         ctx->cluster_order_n = n;
         sorted_ids = vin;
-        // Sizes and segment offsets come from the sorted keys: no counting pass over the assignments.
-        hipLaunchKernelGGL(segment_bounds_kernel, dim3((unsigned) ((n + 1 + 255) / 256)), dim3(256), 0, ctx->stream, kin, n,
-                           (uint32_t) k, offsets);
-        SKM_HIP_TRY(hipGetLastError());
+        // Sizes and segment offsets come from the sorted keys: no counting pass over the assignments.  The scatter of
+        // a one-pass sort has written them already.
+        if (passes > 1) {
+            hipLaunchKernelGGL(segment_bounds_kernel, dim3((unsigned) ((n + 1 + 255) / 256)), dim3(256), 0, ctx->stream, kin, n,
+                               (uint32_t) k, offsets);
+            SKM_HIP_TRY(hipGetLastError());
+        }
     } else {
         sorted_ids = vals_a;
         ctx->cluster_order = nullptr;
@@ -487,8 +509,33 @@ int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size
     SKM_REQUIRE(ctx && d_sums && d_sizes, "null argument");
     if (k == 0) return SKM_OK;
     ScopedStage st(ctx, "consolidate/splitting");
-    hipLaunchKernelGGL(scale_by_size_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_sums, d_sizes, k, d);
+    hipLaunchKernelGGL(scale_by_size_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_sums, d_sizes, k, d,
+                       (uint32_t*) nullptr);
     return check_hip(hipGetLastError(), "scale_by_size_kernel launch");
+}
+
+int skm_scale_by_size_fetch(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d, uint32_t* h_sizes) {
+    SKM_REQUIRE(ctx && d_sums && d_sizes && h_sizes, "null argument");
+    if (k == 0) return SKM_OK;
+    // Up to a few thousand clusters the kernel leaves a copy of the sizes in pinned host memory on its way (one
+    // 4-byte write per cluster); beyond that one copy operation moves them.
+    uint32_t* mirror = nullptr;
+    size_t mirror_entries = 0;
+    SKM_TRY(pinned_sizes(ctx, &mirror, &mirror_entries));
+    if (k > mirror_entries) mirror = nullptr;
+    {
+        ScopedStage st(ctx, "consolidate/splitting");
+        hipLaunchKernelGGL(scale_by_size_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_sums, d_sizes, k, d, mirror);
+        SKM_TRY(check_hip(hipGetLastError(), "scale_by_size_kernel launch"));
+    }
+    if (mirror) {
+        SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+        std::memcpy(h_sizes, mirror, k * sizeof(uint32_t));
+        return SKM_OK;
+    }
+    SKM_HIP_TRY(hipMemcpyAsync(h_sizes, d_sizes, k * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return SKM_OK;
 }
 
 int skm_normalize_rows(skm_ctx* ctx, float* d_c, size_t k, size_t d) {
@@ -538,10 +585,30 @@ int skm_edit_rows(skm_ctx* ctx, float* d_c, size_t d, const uint32_t* h_ops, siz
         std::vector<size_t> cursor(first.begin(), first.end() - 1);
         for (size_t o = 0; o < n_ops; ++o) std::memcpy(&ordered[4 * cursor[round[o]]++], h_ops + 4 * o, 4 * sizeof(uint32_t));
     }
-    void* ws = nullptr;
-    SKM_TRY(workspace(ctx, 2, n_ops * 4 * sizeof(uint32_t), &ws));
-    SKM_HIP_TRY(hipMemcpyAsync(ws, ordered.data(), n_ops * 4 * sizeof(uint32_t), hipMemcpyHostToDevice, ctx->stream));
-    SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));  // `ordered` is released on return
+    // The kernels read the edits from pinned host memory, a ring the context owns: no copy operation and no wait.  A
+    // call that does not fit behind the previous ones starts over at the front after a wait for the stream; a call
+    // larger than the ring goes through device memory.
+    const void* ws = nullptr;
+    const size_t bytes = n_ops * 4 * sizeof(uint32_t);
+    void* ring = nullptr;
+    size_t ring_bytes = 0;
+    SKM_TRY(host_ring(ctx, &ring, &ring_bytes));
+    if (bytes <= ring_bytes) {
+        if (ctx->h_ring_used + bytes > ring_bytes) {
+            SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
+            ctx->h_ring_used = 0;
+        }
+        void* at = (char*) ring + ctx->h_ring_used;
+        std::memcpy(at, ordered.data(), bytes);
+        ctx->h_ring_used += (bytes + 63) / 64 * 64;
+        ws = at;
+    } else {
+        void* dev = nullptr;
+        SKM_TRY(workspace(ctx, 2, bytes, &dev));
+        SKM_HIP_TRY(hipMemcpyAsync(dev, ordered.data(), bytes, hipMemcpyHostToDevice, ctx->stream));
+        SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));  // `ordered` is released on return
+        ws = dev;
+    }
     for (int r = 0; r < n_rounds; ++r) {
         const size_t count = first[r + 1] - first[r];
         hipLaunchKernelGGL(edit_rows_kernel, dim3((unsigned) count), dim3(256), 0, ctx->stream, d_c, d,

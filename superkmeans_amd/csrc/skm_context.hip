@@ -118,18 +118,55 @@ int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out) {
     return SKM_OK;
 }
 
-int pinned(skm_ctx* ctx, size_t bytes, void** out) {
-    if (ctx->h_pinned_bytes < bytes) {
-        if (ctx->h_pinned) {
-            SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
-            SKM_HIP_TRY(hipHostFree(ctx->h_pinned));
-            ctx->h_pinned = nullptr;
-            ctx->h_pinned_bytes = 0;
-        }
-        SKM_HIP_TRY(hipHostMalloc(&ctx->h_pinned, bytes, hipHostMallocDefault));
-        ctx->h_pinned_bytes = bytes;
+// One pinned host block per context, allocated at first use (pinned allocations are slow and every helper context of
+// a hierarchical Train has its own): result slots, then the copy of the cluster sizes, then the ring of row edits.
+constexpr size_t PINNED_SLOTS_BYTES = 256;
+constexpr size_t PINNED_SIZES_BYTES = size_t(16384) * sizeof(uint32_t);
+constexpr size_t PINNED_RING_BYTES = size_t(256) << 10;
+
+static int pinned_block(skm_ctx* ctx) {
+    if (!ctx->h_pinned) {
+        const size_t total = PINNED_SLOTS_BYTES + PINNED_SIZES_BYTES + PINNED_RING_BYTES;
+        SKM_HIP_TRY(hipHostMalloc(&ctx->h_pinned, total, hipHostMallocDefault));
+        ctx->h_pinned_bytes = total;
+        ctx->h_ring_used = 0;
     }
+    return SKM_OK;
+}
+
+int pinned(skm_ctx* ctx, size_t bytes, void** out) {
+    if (bytes > PINNED_SLOTS_BYTES) return set_error(SKM_ERR_INVALID, "pinned: %zu bytes of result slots requested", bytes);
+    SKM_TRY(pinned_block(ctx));
     *out = ctx->h_pinned;
+    return SKM_OK;
+}
+
+int pinned_sizes(skm_ctx* ctx, uint32_t** out, size_t* out_entries) {
+    SKM_TRY(pinned_block(ctx));
+    *out = reinterpret_cast<uint32_t*>((char*) ctx->h_pinned + PINNED_SLOTS_BYTES);
+    *out_entries = PINNED_SIZES_BYTES / sizeof(uint32_t);
+    return SKM_OK;
+}
+
+int host_ring(skm_ctx* ctx, void** out, size_t* out_bytes) {
+    SKM_TRY(pinned_block(ctx));
+    *out = (char*) ctx->h_pinned + PINNED_SLOTS_BYTES + PINNED_SIZES_BYTES;
+    *out_bytes = PINNED_RING_BYTES;
+    return SKM_OK;
+}
+
+int reduction_counter(skm_ctx* ctx, uint32_t** out) {
+    if (!ctx->d_reduction_counter) {
+        void* p = nullptr;
+        SKM_TRY(device_alloc(ctx->device, 256, &p));
+        const hipError_t e = hipMemsetAsync(p, 0, 256, ctx->stream);
+        if (e != hipSuccess) {
+            (void) device_release(ctx->device, p);
+            return check_hip(e, "hipMemsetAsync");
+        }
+        ctx->d_reduction_counter = (uint32_t*) p;
+    }
+    *out = ctx->d_reduction_counter;
     return SKM_OK;
 }
 
@@ -244,6 +281,7 @@ int skm_ctx_destroy(skm_ctx* ctx) {
     for (auto e : ctx->event_pool) (void) hipEventDestroy(e);
     for (int i = 0; i < skm_ctx::WS_SLOTS; ++i)
         if (ctx->ws[i]) (void) device_release(ctx->device, ctx->ws[i]);
+    if (ctx->d_reduction_counter) (void) device_release(ctx->device, ctx->d_reduction_counter);
     if (ctx->h_pinned) (void) hipHostFree(ctx->h_pinned);
     if (ctx->copy_stream) {
         (void) hipStreamSynchronize(ctx->copy_stream);

@@ -39,7 +39,12 @@ struct skm_ctx {
     // fetched them first.  Any permutation of the points gives the same results.
     const uint32_t* cluster_order = nullptr;
     size_t cluster_order_n = 0;
-    // Small pinned host buffer for scalar results.
+    // "Blocks done" counter of the single-launch reductions (device memory, zero between launches).
+    uint32_t* d_reduction_counter = nullptr;
+    // One pinned host block: result slots of the reductions, a copy of the cluster sizes written by the kernel that
+    // scales the sums, and a ring that kernels read small host-made tables from (row edits); h_ring_used is the
+    // ring's fill.
+    size_t h_ring_used = 0;
     void* h_pinned = nullptr;
     size_t h_pinned_bytes = 0;
     // Address, on this context's device, of the library's static scratch array (skm_assign_full_noalloc).
@@ -79,6 +84,9 @@ int device_release(int device, void* ptr);
 // Returns a scratch buffer of at least `bytes` for slot `slot` (grow-only).
 int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out);
 int pinned(skm_ctx* ctx, size_t bytes, void** out);
+int reduction_counter(skm_ctx* ctx, uint32_t** out);
+int host_ring(skm_ctx* ctx, void** out, size_t* out_bytes);
+int pinned_sizes(skm_ctx* ctx, uint32_t** out, size_t* out_entries);
 
 // RAII device timer for one profiler scope; no-op unless profiling is enabled.
 class ScopedStage {

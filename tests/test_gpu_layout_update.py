@@ -34,7 +34,10 @@ def test_pdxify_rejects_bad_split(capi, ctx):
                                             (40000, 1024, 9, 4), (50000, 512, 20, 2),
                                             # ragged column groups of the row-sum kernel: 33 and 5 float4 lanes, 20 and 200
                                             # single-float lanes (the last wavefront of a centroid is partly idle)
-                                            (30000, 132, 3000, 2), (20000, 20, 3000, 1), (5000, 20, 10, 1), (30000, 200, 600, 3)])
+                                            (30000, 132, 3000, 2), (20000, 20, 3000, 1), (5000, 20, 10, 1), (30000, 200, 600, 3),
+                                            # one sort pass with every digit a centroid (k = 256) and all but one (255):
+                                            # the segment offsets come from the scatter kernel there
+                                            (6000, 96, 256, 2), (4001, 64, 255, 1), (39062, 128, 256, 4)])
 def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
     g = np.random.default_rng(n + d)
     X = g.standard_normal((n, d)).astype(np.float32)
@@ -48,7 +51,15 @@ def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
     assert np.array_equal(sizes, rz)
     assert np.array_equal(sizes, np.bincount(a, minlength=k).astype(np.uint32))
     assert np.array_equal(sums, rs)  # same summation order as the reference -> identical bits
-    capi.check(ctx.lib.skm_scale_by_size(ctx.handle, dS.ptr, dZ.ptr, k, d))
+    if (n + k) % 2 == 0:
+        capi.check(ctx.lib.skm_scale_by_size(ctx.handle, dS.ptr, dZ.ptr, k, d))
+    else:
+        # the variant that hands the sizes to the host on its way (a pinned copy up to 16,384 clusters, a copy beyond)
+        import ctypes
+        fetched = np.full(k, 0xffffffff, dtype=np.uint32)
+        capi.check(ctx.lib.skm_scale_by_size_fetch(ctx.handle, dS.ptr, dZ.ptr, k, d,
+                                                   fetched.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))))
+        assert np.array_equal(fetched, rz)
     means = dS.download()
     rm, _ = oracle.update_centroids(X, a, k, scale=True, n_threads=nthreads)
     assert np.array_equal(means, rm)
