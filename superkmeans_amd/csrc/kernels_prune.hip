@@ -76,6 +76,29 @@ inline unsigned die_striped_groups(int n, int waves_per_group) {
     return (groups + 7) / 8 * 8;
 }
 
+// The same pointer, said to be equal in all lanes (it is: it derives from the batch and block indices) and to point to
+// global memory (an address built from integers is otherwise taken for a flat one, whose loads are waited for all at
+// once): the compiler then keeps it in scalar registers and a gather needs only its 32-bit lane offset in a vector
+// register.
+typedef const char __attribute__((address_space(1)))* global_bytes_t;
+typedef float gather4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ global_bytes_t uniform_pointer(const void* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t) v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t) (v >> 32));
+    return reinterpret_cast<global_bytes_t>(((uint64_t) hi << 32) | lo);
+}
+// Four floats at byte offset `off` of a block (16-byte load when VEC).
+template <bool VEC>
+__device__ __forceinline__ float4 gather4(global_bytes_t base, uint32_t off) {
+    if (VEC) {
+        const gather4_t g = *reinterpret_cast<const gather4_t __attribute__((address_space(1)))*>(base + off);
+        return make_float4(g.x, g.y, g.z, g.w);
+    }
+    const float __attribute__((address_space(1)))* f = reinterpret_cast<const float __attribute__((address_space(1)))*>(base + off);
+    return make_float4(f[0], f[1], f[2], f[3]);
+}
+
 // Four consecutive floats of a point row (16-byte load when rows are aligned).
 template <bool VEC>
 __device__ __forceinline__ float4 load_x4(const float* p) {
@@ -199,19 +222,14 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
             // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.  Slots past
             // the last survivor read the pad (position 0) and their sums land in the pad.
             if (lane < LIST_PAD) pos[cnt + lane] = 0;
-            const char* blk_bytes = reinterpret_cast<const char*>(blk);
+            const global_bytes_t blk_bytes = uniform_pointer(blk);
             const uint32_t lane_bytes = (uint32_t) sub * 16u;
             for (int s0 = 0; s0 < cnt; s0 += 32) {
                 float4 cv[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) {
                     const uint32_t cpos = pos[s0 + 4 * u + grp];
-                    const float* cb = reinterpret_cast<const float*>(blk_bytes + ((cpos << 8) | lane_bytes));
-                    if (VEC) {
-                        cv[u] = *reinterpret_cast<const float4*>(cb);
-                    } else {
-                        cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
-                    }
+                    cv[u] = gather4<VEC>(blk_bytes, (cpos << 8) | lane_bytes);
                 }
                 float mine = 0.0f;
 #pragma unroll
@@ -519,19 +537,14 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
                 // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.  Slots past
                 // the last survivor read the pad (position 0) and their sums land in the pad.
                 if (lane < LIST_PAD) pos[cnt + lane] = 0;
-                const char* blk_bytes = reinterpret_cast<const char*>(blk);
+                const global_bytes_t blk_bytes = uniform_pointer(blk);
                 const uint32_t lane_bytes = (uint32_t) sub * 16u;
                 for (int s0 = 0; s0 < cnt; s0 += 32) {
                     float4 cv[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) {
                         const uint32_t cpos = pos[s0 + 4 * u + grp];
-                        const float* cb = reinterpret_cast<const float*>(blk_bytes + ((cpos << 8) | lane_bytes));
-                        if (VEC) {
-                            cv[u] = *reinterpret_cast<const float4*>(cb);
-                        } else {
-                            cv[u] = make_float4(cb[0], cb[1], cb[2], cb[3]);
-                        }
+                        cv[u] = gather4<VEC>(blk_bytes, (cpos << 8) | lane_bytes);
                     }
                     // all 16 lanes of a group hold the sum of each of its eight survivors: lane u of the group keeps
                     // the u-th and the first eight lanes add theirs in one go
