@@ -44,13 +44,13 @@ PEAK_HBM_GBPS = 8000.0
 # not profiled.  They describe the build the summaries were taken with; a change to a kernel needs a new profile run.
 #   profiles/gemm_argmin_kernel_assign_n1M_d1024_k10k_hbm_traffic.md: the two gemm_argmin_kernel launches of an Assign pass
 MEASURED_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000): int(((31_470_719 + 2_006_672) * 1.943 + 609_375 + 7_812) * 1024),
+    (1_000_000, 1024, 10_000): int(((31_547_474 + 2_006_025) * 1.943 + 609_375 + 7_812) * 1024),
 }
 #   same file: every seed_distance_kernel, prune_list_kernel and prune_kernel launch of one Train of (n, d, k, iterations)
 MEASURED_PRUNE_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000, 10): int((50_265_137 * 1.943 + 1_471_834) * 1024),
+    (1_000_000, 1024, 10_000, 10): int((49_192_385 * 1.943 + 1_472_410) * 1024),
     # profiles/train_n2M_d1536_k4096_kernel_stats_list_walk_traffic.md
-    (2_000_000, 1536, 4_096, 10): int((845_534_958 * 1.943 + 2_864_203) * 1024),
+    (2_000_000, 1536, 4_096, 10): int((844_550_017 * 1.943 + 2_873_152) * 1024),
 }
 
 
@@ -239,7 +239,7 @@ def main():
             stage["prune"]["measured_bytes"] = measured
             stage["prune"]["measured_frac"] = round(measured / (stage["prune"]["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4) \
                 if measured else None
-            stage["prune"]["bound_note"] = "bound by instruction issue and cache gathers before HBM: see ns_per_pair_block"
+            stage["prune"]["bound_note"] = "dependent steps on short survivor lists, instruction issue and cache gathers before HBM: see ns_per_pair_block"
         if hierarchical:
             train["phases"] = {name: {"iterations": len(v), "final_objective": (v[-1].objective if v and name != "fineclustering" else None)}
                                for name, v in phase_stats.items()}
