@@ -8,14 +8,14 @@ namespace skm {
 // chunk of up to 1024 centroids the first vertical_d columns become dimension-major.  32 x 32 tiles
 // are staged through LDS so that both the row-major reads and the dimension-major writes are
 // coalesced.
-__global__ __launch_bounds__(256) void pdx_vertical_kernel(
-    const float* __restrict__ in, size_t k, size_t d, size_t V, float* __restrict__ out
+__device__ __forceinline__ void pdx_vertical_tile(
+    const float* __restrict__ in, size_t k, size_t d, size_t V, float* __restrict__ out, size_t tile_x, size_t tile_y,
+    size_t chunk
 ) {
     __shared__ float tile[32][33];
-    const size_t chunk = blockIdx.z;
     const size_t base_row = chunk * SKM_Y_BATCH_SIZE;
     const size_t m = (k - base_row) < SKM_Y_BATCH_SIZE ? (k - base_row) : SKM_Y_BATCH_SIZE;
-    const size_t r0 = (size_t) blockIdx.y * 32, c0 = (size_t) blockIdx.x * 32;
+    const size_t r0 = tile_y * 32, c0 = tile_x * 32;
     if (r0 >= m) return;
     const float* src = in + base_row * d;
     float* dst = out + base_row * d;
@@ -33,10 +33,9 @@ __global__ __launch_bounds__(256) void pdx_vertical_kernel(
 
 // Horizontal part (pdx/layout.h:186-192,216-222): 64-wide row-major blocks, one after the other.
 // Also emits the dense copy of the first V columns (superkmeans.h:1206-1212) when aux != nullptr.
-__global__ __launch_bounds__(256) void pdx_horizontal_kernel(
-    const float* __restrict__ in, size_t k, size_t d, size_t V, float* __restrict__ out, float* __restrict__ aux
+__device__ __forceinline__ void pdx_horizontal_row(
+    const float* __restrict__ in, size_t k, size_t d, size_t V, float* __restrict__ out, float* __restrict__ aux, size_t row
 ) {
-    const size_t row = blockIdx.x;  // global centroid index
     const size_t chunk = row / SKM_Y_BATCH_SIZE;
     const size_t base_row = chunk * SKM_Y_BATCH_SIZE;
     const size_t m = (k - base_row) < SKM_Y_BATCH_SIZE ? (k - base_row) : SKM_Y_BATCH_SIZE;
@@ -50,6 +49,21 @@ __global__ __launch_bounds__(256) void pdx_horizontal_kernel(
     if (aux) {
         float* a = aux + row * V;
         for (size_t j = threadIdx.x; j < V; j += blockDim.x) a[j] = src[j];
+    }
+}
+
+// Both parts in one launch: the first vertical_tiles workgroups (tile column fastest, then tile row, then chunk) transpose
+// tiles of the vertical part, the next horizontal_rows take one centroid each.
+__global__ __launch_bounds__(256) void pdxify_kernel(
+    const float* __restrict__ in, size_t k, size_t d, size_t V, float* __restrict__ out, float* __restrict__ aux,
+    uint32_t tiles_x, uint32_t vertical_tiles
+) {
+    if (blockIdx.x < vertical_tiles) {
+        constexpr uint32_t TILES_Y = SKM_Y_BATCH_SIZE / 32;
+        const uint32_t b = blockIdx.x;
+        pdx_vertical_tile(in, k, d, V, out, b % tiles_x, (b / tiles_x) % TILES_Y, b / (tiles_x * TILES_Y));
+    } else {
+        pdx_horizontal_row(in, k, d, V, out, aux, blockIdx.x - vertical_tiles);
     }
 }
 
@@ -95,14 +109,13 @@ int skm_pdxify(skm_ctx* ctx, const float* d_c, size_t k, size_t d, size_t vertic
     ScopedStage st(ctx, "consolidate/pdxify");
     const size_t n_chunks = (k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE;
     SKM_REQUIRE(n_chunks <= 65535, "too many centroids");
-    dim3 gv((unsigned) ((vertical_d + 31) / 32), SKM_Y_BATCH_SIZE / 32, (unsigned) n_chunks);
-    hipLaunchKernelGGL(pdx_vertical_kernel, gv, dim3(256), 0, ctx->stream, d_c, k, d, vertical_d, d_pdx);
-    SKM_HIP_TRY(hipGetLastError());
-    if (d > vertical_d || d_aux) {
-        hipLaunchKernelGGL(pdx_horizontal_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_c, k, d, vertical_d, d_pdx, d_aux);
-        SKM_HIP_TRY(hipGetLastError());
-    }
-    return SKM_OK;
+    const uint32_t tiles_x = (uint32_t) ((vertical_d + 31) / 32);
+    const size_t vertical_tiles = (size_t) tiles_x * (SKM_Y_BATCH_SIZE / 32) * n_chunks;
+    const size_t horizontal_rows = (d > vertical_d || d_aux) ? k : 0;
+    SKM_REQUIRE(vertical_tiles + horizontal_rows <= 0x7fffffffULL, "too many centroids for one launch");
+    hipLaunchKernelGGL(pdxify_kernel, dim3((unsigned) (vertical_tiles + horizontal_rows)), dim3(256), 0, ctx->stream, d_c, k, d,
+                       vertical_d, d_pdx, d_aux, tiles_x, (uint32_t) vertical_tiles);
+    return check_hip(hipGetLastError(), "pdxify_kernel launch");
 }
 
 int skm_gather_rows(skm_ctx* ctx, const float* d_x, size_t d, const uint64_t* d_index, size_t m, float* d_out,

@@ -326,9 +326,11 @@ template <bool VEC>
 __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
     const float* __restrict__ x, const float* __restrict__ c, const uint32_t* __restrict__ idx, int n, int d,
     const float* __restrict__ ratios, int partial_d, float* __restrict__ best0, float* __restrict__ thr0,
-    const uint32_t* __restrict__ order
+    const uint32_t* __restrict__ order, uint32_t* __restrict__ zero_this
 ) {
     const int lane = threadIdx.x & 63;
+    // the first launch of a search also clears the count of overflowing points that later kernels add to
+    if (zero_this && blockIdx.x == 0 && threadIdx.x == 0) *zero_this = 0u;
     const int p = point_of_wave(order, n, PRUNE_WAVES);
     if (p < 0) return;
     const float* xq = x + (int64_t) p * d;
@@ -398,6 +400,9 @@ struct PruneListArgs {
     uint32_t* not_pruned;
     unsigned long long* stage_pairs;
     const uint32_t* order;        // null, or the sequence in which the wavefronts take the points
+    uint64_t* over_ids;           // ids (id_offset + point) of the points whose list overflowed, appended here
+    uint32_t* n_over;             // their count
+    uint64_t id_offset;
     int n, k, d, vertical_d, partial_d;
 };
 
@@ -415,7 +420,10 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     if (p < 0) return;
     float* parts = s_parts[wave];
     const uint32_t n_cand = a.cand_count[p];
-    if (n_cand > a.cap) return;  // handled densely by the caller
+    if (n_cand > a.cap) {  // handled densely by the caller, who finds the point in the list of overflowing ones
+        if (lane == 0) a.over_ids[atomicAdd(a.n_over, 1u)] = a.id_offset + (uint64_t) p;
+        return;
+    }
     uint16_t* pos = s_pos[wave];
     float* acc = s_acc[wave];
     const int d = a.d, V = a.vertical_d, dp = a.partial_d;
@@ -635,28 +643,6 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     }
 }
 
-// Appends the ids (id_offset + chunk-local index) of the points whose candidate list overflowed.
-// With a visiting order the points are examined in that order, so that neighbours in the list of overflowing points
-// tend to be neighbours in the order (the list is only as ordered as the atomics of concurrently running wavefronts
-// leave it; its order changes where the dense redo finds its centroid blocks, not what it computes).
-__global__ __launch_bounds__(256) void collect_overflow_kernel(
-    const uint32_t* __restrict__ cand_count, int n, uint32_t cap, uint64_t id_offset, uint64_t* __restrict__ ids,
-    uint32_t* __restrict__ n_over, const uint32_t* __restrict__ order
-) {
-    const int slot = blockIdx.x * blockDim.x + threadIdx.x;
-    if (slot >= n) return;
-    const uint32_t i = order ? order[slot] : (uint32_t) slot;
-    const bool over = cand_count[i] > cap;
-    // one atomic per wavefront: its overflowing points take consecutive entries in lane order
-    const unsigned long long mask = __ballot(over);
-    if (mask == 0) return;
-    const int lane = threadIdx.x & 63;
-    uint32_t base = 0;
-    if (lane == __ffsll((long long) mask) - 1) base = atomicAdd(n_over, (uint32_t) __popcll(mask));
-    base = (uint32_t) __shfl((int) base, __ffsll((long long) mask) - 1);
-    if (over) ids[base + (uint32_t) __popcll(mask & ((1ull << lane) - 1ull))] = id_offset + (uint64_t) i;
-}
-
 __global__ __launch_bounds__(256) void gather_u32_kernel(const uint32_t* __restrict__ in, const uint64_t* __restrict__ ids, int m, uint32_t* __restrict__ out) {
     const int j = blockIdx.x * blockDim.x + threadIdx.x;
     if (j < m) out[j] = in[ids[j]];
@@ -668,24 +654,27 @@ __global__ __launch_bounds__(256) void scatter_u32_kernel(const uint32_t* __rest
 }
 
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
-                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order) {
+                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order,
+                         uint32_t* zero_this) {
     if (n <= 0) return SKM_OK;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(c) % 16 == 0);
     dim3 grid(die_striped_groups(n, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (vec)
-        hipLaunchKernelGGL(seed_distance_kernel<true>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order);
+        hipLaunchKernelGGL(seed_distance_kernel<true>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order, zero_this);
     else
-        hipLaunchKernelGGL(seed_distance_kernel<false>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order);
+        hipLaunchKernelGGL(seed_distance_kernel<false>, grid, block, 0, ctx->stream, x, c, idx, n, d, ratios, partial_d, best0, thr0, order, zero_this);
     return check_hip(hipGetLastError(), "seed_distance_kernel launch");
 }
 
 int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
-                      unsigned long long* d_stage_pairs, const uint32_t* order) {
+                      unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
+                      uint64_t id_offset) {
     if (n_chunk <= 0) return SKM_OK;
     PruneListArgs a;
     a.order = order;
+    a.over_ids = over_ids; a.n_over = n_over; a.id_offset = id_offset;
     a.cand = cand; a.cand_count = cand_count; a.cap = cap; a.best0 = best0; a.x = x; a.pdx = pdx; a.aux = aux;
     a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
@@ -700,14 +689,6 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     else
         hipLaunchKernelGGL((prune_list_kernel<false, false>), grid, block, 0, ctx->stream, a);
     return check_hip(hipGetLastError(), "prune_list_kernel launch");
-}
-
-int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
-                            uint64_t* ids, uint32_t* n_over, const uint32_t* order) {
-    if (n <= 0) return SKM_OK;
-    hipLaunchKernelGGL(collect_overflow_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, cand_count, n, cap,
-                       id_offset, ids, n_over, order);
-    return check_hip(hipGetLastError(), "collect_overflow_kernel launch");
 }
 
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out) {

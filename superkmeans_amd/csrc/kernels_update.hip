@@ -313,7 +313,8 @@ constexpr int REDUCE_BLOCKS = 512;
 template <int MODE>  // 0: sum a[i]; 1: sum (a[i]-b[i])^2; 2: sum of uint32 a[i] (as exact integers)
 __global__ __launch_bounds__(256) void reduce_kernel(
     const float* __restrict__ a, const float* __restrict__ b, size_t n, double* __restrict__ partial,
-    uint32_t* __restrict__ counter, double* __restrict__ out
+    uint32_t* __restrict__ counter, double* __restrict__ out, const uint32_t* __restrict__ word_in,
+    uint32_t* __restrict__ word_out
 ) {
     __shared__ double s[256];
     __shared__ uint32_t s_done;
@@ -352,6 +353,7 @@ __global__ __launch_bounds__(256) void reduce_kernel(
     if (threadIdx.x == 0) {
         out[0] = s[0];
         *counter = 0u;
+        if (word_in) *word_out = *word_in;  // a device word the host wants with the same wait (earlier kernels wrote it)
     }
 }
 
@@ -368,18 +370,19 @@ static int result_slot(skm_ctx* ctx, int slot, double** out) {
 }
 
 // Queues the reduction; the result is in *h_slot once the stream has been waited for.
-static int reduce_enqueue(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_slot) {
+static int reduce_enqueue(skm_ctx* ctx, int mode, const float* a, const float* b, size_t n, double* h_slot,
+                          const uint32_t* d_word = nullptr, uint32_t* h_word = nullptr) {
     void* ws = nullptr;
     SKM_TRY(workspace(ctx, 3, (REDUCE_BLOCKS + 8) * sizeof(double), &ws));
     double* partial = (double*) ws;
     uint32_t* counter = nullptr;
     SKM_TRY(reduction_counter(ctx, &counter));
     if (mode == 0)
-        hipLaunchKernelGGL(reduce_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
+        hipLaunchKernelGGL(reduce_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     else if (mode == 1)
-        hipLaunchKernelGGL(reduce_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
+        hipLaunchKernelGGL(reduce_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     else
-        hipLaunchKernelGGL(reduce_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot);
+        hipLaunchKernelGGL(reduce_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     return check_hip(hipGetLastError(), "reduce_kernel launch");
 }
 
@@ -396,9 +399,10 @@ int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_
     return reduce_to_host(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, h_out);
 }
 
-int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot) {
+int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot, const uint32_t* d_word,
+                           uint32_t* h_word) {
     SKM_TRY(result_slot(ctx, SLOT_NOT_PRUNED, h_slot));
-    return reduce_enqueue(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, *h_slot);
+    return reduce_enqueue(ctx, 2, reinterpret_cast<const float*>(a), nullptr, n, *h_slot, d_word, h_word);
 }
 
 int overflow_count_slot(skm_ctx* ctx, uint32_t** h_slot) {

@@ -143,13 +143,13 @@ int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const
                                       uint32_t* cand_count, uint2* cand, uint32_t cap);
 // `order`: null, or a permutation of the n points giving the sequence in which wavefronts take them.
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
-                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order);
+                         const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order,
+                         uint32_t* zero_this);
 int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
-                      unsigned long long* d_stage_pairs, const uint32_t* order);
-int launch_collect_overflow(skm_ctx* ctx, const uint32_t* cand_count, int n, uint32_t cap, uint64_t id_offset,
-                            uint64_t* ids, uint32_t* n_over, const uint32_t* order);
+                      unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
+                      uint64_t id_offset);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 

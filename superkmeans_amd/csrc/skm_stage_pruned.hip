@@ -17,7 +17,8 @@
 
 namespace skm {
 int reduce_u32_sum_to_host(skm_ctx* ctx, const uint32_t* a, size_t n, double* h_out);
-int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot);
+int reduce_u32_sum_enqueue(skm_ctx* ctx, const uint32_t* a, size_t n, double** h_slot, const uint32_t* d_word,
+                           uint32_t* h_word);
 int overflow_count_slot(skm_ctx* ctx, uint32_t** h_slot);
 }
 
@@ -123,7 +124,6 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     float* d_thr0 = d_best0 + cn;
     uint32_t* d_cand_count = (uint32_t*) (d_thr0 + cn);
     uint32_t* d_n_over = d_cand_count + cn;
-    SKM_TRY(skm_fill_u32(ctx, d_n_over, 0u, 1));
 
     // The order the last centroid update left, when it covers exactly these points and they are one chunk.
     const uint32_t* order = (chunk >= n && ctx->cluster_order_n == n) ? ctx->cluster_order : nullptr;
@@ -135,7 +135,7 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         {
             ScopedStage st(ctx, "search/seed");
             SKM_TRY(launch_seed_distance(ctx, xc, d_c, d_inout_idx + i0, (int) m, (int) d, d_ratios, (int) partial_d,
-                                         d_best0, d_thr0, order));
+                                         d_best0, d_thr0, order, i0 == 0 ? d_n_over : (uint32_t*) nullptr));
         }
         {
             ScopedStage st(ctx, "search/blas");
@@ -149,12 +149,11 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
                 SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
                                                d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
         }
-        SKM_TRY(launch_collect_overflow(ctx, d_cand_count, (int) m, cap, (uint64_t) i0, d_over_ids, d_n_over, order));
         {
             ScopedStage st(ctx, "search/pdx");
             SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
                                       (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
-                                      d_out_dist + i0, d_counts + i0, stage_arg, order));
+                                      d_out_dist + i0, d_counts + i0, stage_arg, order, d_over_ids, d_n_over, (uint64_t) i0));
         }
     }
     // Points whose list overflowed (loose seeds, or points with no centroid nearby): one dense redo for
@@ -162,10 +161,14 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     // per-point counts is queued before the number of overflowing points is known and both arrive with one wait;
     // it is taken again only if a redo changed some counts.
     double* h_not_pruned = nullptr;
-    if (h_out_not_pruned) SKM_TRY(reduce_u32_sum_enqueue(ctx, d_counts, n, &h_not_pruned));
     uint32_t* h_n_over = nullptr;
     SKM_TRY(overflow_count_slot(ctx, &h_n_over));
-    SKM_HIP_TRY(hipMemcpyAsync(h_n_over, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    if (h_out_not_pruned) {
+        // the reduction's last block also leaves the number of overflowing points in its host slot
+        SKM_TRY(reduce_u32_sum_enqueue(ctx, d_counts, n, &h_not_pruned, d_n_over, h_n_over));
+    } else {
+        SKM_HIP_TRY(hipMemcpyAsync(h_n_over, d_n_over, sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    }
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
     const size_t mo = *(volatile uint32_t*) h_n_over;
     if (mo > 0) {
