@@ -16,11 +16,12 @@
 namespace skm {
 
 constexpr int SORT_THREADS = 256;
-// Elements per workgroup and pass.  Smaller tiles give more workgroups but shorter runs of equal digits per tile: with a
-// million keys the scatter of a pass over random low digits writes 16-byte runs at 1,024 and takes longer than at
-// 4,096.  A sort of a few ten thousand keys (a fine clustering) is a matter of latency instead: ten workgroups of
-// sixteen rounds each, so there the small tile is the faster one.
-constexpr int SORT_TILE = 4096, SORT_TILE_FEW_KEYS = 1024;
+// Elements per workgroup and pass.  Smaller tiles give more workgroups (a workgroup is four wavefronts whose rounds are
+// separated by barriers, so a compute unit needs several to hide their latencies) but shorter runs of equal digits per
+// tile and a longer table of per-tile digit counts.  Measured with a million 14-bit keys (7 + 7 bits), both passes
+// together: 4,096 keys per tile 64 us, 2,048 58 us, 1,024 65 us (there the scans of the 977-entry rows take 10 us each).
+// A sort of a few ten thousand keys (a fine clustering) is a matter of latency: there the smallest tile is the fastest.
+constexpr int SORT_TILE = 2048, SORT_TILE_FEW_KEYS = 1024;  // multiples of the scatter's round of 1,024 elements
 constexpr size_t SORT_FEW_KEYS = size_t(1) << 18;
 constexpr int RADIX = 256;
 
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(256) void segment_bounds_kernel(
 // First step of a radix pass: digit histogram of one tile, stored digit-major ([digit][tile]) so that every digit's
 // counts over the tiles are one contiguous row for digit_rows_scan_kernel.
 __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
-    const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t n_tiles, int tile, uint32_t* __restrict__ hist
+    const uint32_t* __restrict__ keys, size_t n, int shift, uint32_t mask, uint32_t n_tiles, int tile, uint32_t* __restrict__ hist
 ) {
     __shared__ uint32_t s_hist[RADIX];
     s_hist[threadIdx.x] = 0;
@@ -81,17 +82,17 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_hist_kernel(
     const size_t t0 = (size_t) blockIdx.x * tile;
     for (int r = 0; r < tile / SORT_THREADS; ++r) {
         const size_t i = t0 + (size_t) r * SORT_THREADS + threadIdx.x;
-        if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & (RADIX - 1)], 1u);
+        if (i < n) atomicAdd(&s_hist[(keys[i] >> shift) & mask], 1u);
     }
     __syncthreads();
     hist[(size_t) threadIdx.x * n_tiles + blockIdx.x] = s_hist[threadIdx.x];
 }
 
-// Third step: stable scatter.  The tile is consumed in rounds of 256 consecutive elements; inside a
-// round the rank of an element among equal digits is (equal digits in earlier wavefronts) +
+// Third step: stable scatter.  The tile is consumed in sub-rounds of 256 consecutive elements; inside a
+// sub-round the rank of an element among equal digits is (equal digits in earlier wavefronts) +
 // (equal digits in lower lanes of its wavefront), the latter from eight ballots.
 __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
-    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift,
+    const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in, size_t n, int shift, uint32_t mask,
     uint32_t n_tiles, int tile, const uint32_t* __restrict__ bases, const uint32_t* __restrict__ totals,
     uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out, int vals_are_iota,
     uint32_t* __restrict__ offsets_out, uint32_t k
@@ -122,42 +123,60 @@ __global__ __launch_bounds__(SORT_THREADS) void radix_scatter_kernel(
             if (k == RADIX && tid == 0) offsets_out[RADIX] = (uint32_t) n;
         }
     }
+    // Rounds of 4 x 256 consecutive elements: the four sub-rounds of a round share its barriers.  s_wave_cnt[w][digit]
+    // holds four byte counters, one per sub-round (a wavefront has at most 64 equal digits in a sub-round).
+    constexpr int SUB = 4;
     const size_t t0 = (size_t) blockIdx.x * tile;
-    for (int r = 0; r < tile / SORT_THREADS; ++r) {
-        const size_t i = t0 + (size_t) r * SORT_THREADS + tid;
-        const bool in = i < n;
+    for (int r = 0; r < tile / (SORT_THREADS * SUB); ++r) {
 #pragma unroll
         for (int w = 0; w < SORT_THREADS / 64; ++w) s_wave_cnt[w][tid] = 0;
         __syncthreads();
-        uint32_t key = 0, val = 0, digit = 0;
-        unsigned long long peers = 0;
-        if (in) {
-            key = keys_in[i];
-            val = vals_are_iota ? (uint32_t) i : vals_in[i];
-            digit = (key >> shift) & (RADIX - 1);
-        }
-        // Lanes holding the same digit (inactive lanes never match an active one).
-        unsigned long long match = __ballot(in);
+        uint32_t key[SUB], val[SUB], digit[SUB], rank_in_wave[SUB];
+        bool in[SUB];
 #pragma unroll
-        for (int b = 0; b < 8; ++b) {
-            const unsigned long long vote = __ballot(in && ((digit >> b) & 1u));
-            match &= ((digit >> b) & 1u) ? vote : ~vote;
+        for (int j = 0; j < SUB; ++j) {
+            const size_t i = t0 + ((size_t) r * SUB + j) * SORT_THREADS + tid;
+            in[j] = i < n;
+            key[j] = val[j] = digit[j] = 0;
+            if (in[j]) {
+                key[j] = keys_in[i];
+                val[j] = vals_are_iota ? (uint32_t) i : vals_in[i];
+                digit[j] = (key[j] >> shift) & mask;
+            }
         }
-        peers = match;
-        const uint32_t rank_in_wave = (uint32_t) __popcll(peers & ((1ull << lane) - 1ull));
-        if (in && rank_in_wave == 0) s_wave_cnt[wave][digit] = (uint32_t) __popcll(peers);
+#pragma unroll
+        for (int j = 0; j < SUB; ++j) {
+            // Lanes holding the same digit (inactive lanes never match an active one).
+            unsigned long long match = __ballot(in[j]);
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                const unsigned long long vote = __ballot(in[j] && ((digit[j] >> b) & 1u));
+                match &= ((digit[j] >> b) & 1u) ? vote : ~vote;
+            }
+            rank_in_wave[j] = (uint32_t) __popcll(match & ((1ull << lane) - 1ull));
+            if (in[j] && rank_in_wave[j] == 0) atomicAdd(&s_wave_cnt[wave][digit[j]], (uint32_t) __popcll(match) << (8 * j));
+        }
         __syncthreads();
-        if (in) {
-            uint32_t before = 0;
-            for (int w = 0; w < wave; ++w) before += s_wave_cnt[w][digit];
-            const uint32_t dst = s_base[digit] + before + rank_in_wave;
-            keys_out[dst] = key;
-            vals_out[dst] = val;
+#pragma unroll
+        for (int j = 0; j < SUB; ++j) {
+            if (in[j]) {
+                // equal digits of the earlier sub-rounds in every wavefront, and of this sub-round in the wavefronts below
+                uint32_t before = 0;
+#pragma unroll
+                for (int w = 0; w < SORT_THREADS / 64; ++w) {
+                    const uint32_t c = s_wave_cnt[w][digit[j]];
+                    before += __builtin_amdgcn_sad_u8(c & ((1u << (8 * j)) - 1u), 0u, 0u);
+                    if (w < wave) before += (c >> (8 * j)) & 0xffu;
+                }
+                const uint32_t dst = s_base[digit[j]] + before + rank_in_wave[j];
+                keys_out[dst] = key[j];
+                vals_out[dst] = val[j];
+            }
         }
         __syncthreads();
         uint32_t add = 0;
 #pragma unroll
-        for (int w = 0; w < SORT_THREADS / 64; ++w) add += s_wave_cnt[w][tid];
+        for (int w = 0; w < SORT_THREADS / 64; ++w) add += __builtin_amdgcn_sad_u8(s_wave_cnt[w][tid], 0u, 0u);
         s_base[tid] += add;
         __syncthreads();
     }
@@ -447,6 +466,8 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         int bits = 0;
         while (bits < 32 && ((k - 1) >> bits) != 0) ++bits;
         const int passes = std::max(1, (bits + 7) / 8);
+        const int digit_bits = passes == 1 ? 8 : (bits + passes - 1) / passes;
+        const uint32_t mask = (1u << digit_bits) - 1u;
         const uint32_t* kin = d_idx;
         const uint32_t* vin = nullptr;
         uint32_t* kout = keys_a;
@@ -458,12 +479,14 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         ctx->cluster_order_n = 0;
         uint32_t* vout = passes == 1 ? (uint32_t*) ws_order : vals_a;
         for (int p = 0; p < passes; ++p) {
-            const int shift = 8 * p;
-            hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, n_tiles, tile, hist);
+            // the key bits are spread evenly over the passes (14 bits: 7 + 7, not 8 + 6): fewer distinct digits in a pass
+            // mean longer runs of equal digits per tile, which the scatter writes as longer contiguous pieces
+            const int shift = digit_bits * p;
+            hipLaunchKernelGGL(radix_hist_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, n, shift, mask, n_tiles, tile, hist);
             SKM_HIP_TRY(hipGetLastError());
             hipLaunchKernelGGL(digit_rows_scan_kernel, dim3(RADIX), dim3(64), 0, ctx->stream, hist, n_tiles, bases, totals);
             SKM_HIP_TRY(hipGetLastError());
-            hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift,
+            hipLaunchKernelGGL(radix_scatter_kernel, dim3(n_tiles), dim3(SORT_THREADS), 0, ctx->stream, kin, vin, n, shift, mask,
                                n_tiles, tile, bases, totals, kout, vout, p == 0 ? 1 : 0,
                                passes == 1 ? offsets : (uint32_t*) nullptr, (uint32_t) k);
             SKM_HIP_TRY(hipGetLastError());
