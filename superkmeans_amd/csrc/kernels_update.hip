@@ -27,30 +27,34 @@ constexpr int RADIX = 256;
 
 // Second step of a radix pass.  The histograms are stored digit-major, so the global base of a (digit, tile) pair is
 // (sum of all smaller digits) + (sum of the same digit over the earlier tiles).  One wavefront per digit scans its own
-// row of tile counts, 64 at a time with shuffles and a running carry, and leaves the digit's total; the scatter
-// kernel adds the 256 totals up by itself.  The 256 rows are scanned side by side instead of one scan over
-// 256 * n_tiles counters by a single workgroup.
+// row of tile counts and leaves the digit's total; the scatter kernel adds the 256 totals up by itself.  The 256 rows
+// are scanned side by side instead of one scan over 256 * n_tiles counters by a single workgroup.  A lane owns a
+// contiguous piece of the row: it adds the piece up (independent loads), one scan over the 64 lane sums gives the
+// piece's base, and a second walk of the piece writes the running bases: one shuffle scan per row, whatever its length.
 __global__ __launch_bounds__(64) void digit_rows_scan_kernel(
     const uint32_t* __restrict__ hist, uint32_t n_tiles, uint32_t* __restrict__ bases, uint32_t* __restrict__ totals
 ) {
     const int lane = threadIdx.x;
     const uint32_t* row = hist + (size_t) blockIdx.x * n_tiles;
     uint32_t* out = bases + (size_t) blockIdx.x * n_tiles;
-    uint32_t carry = 0;
-#pragma unroll 4
-    for (uint32_t base = 0; base < n_tiles; base += 64) {
-        const uint32_t i = base + lane;
-        const uint32_t v = i < n_tiles ? row[i] : 0u;
-        uint32_t incl = v;
+    const uint32_t piece = (n_tiles + 63) / 64;
+    const uint32_t from = min((uint32_t) lane * piece, n_tiles), to = min(from + piece, n_tiles);
+    uint32_t sum = 0;
+#pragma unroll 8
+    for (uint32_t i = from; i < to; ++i) sum += row[i];
+    uint32_t incl = sum;
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const uint32_t t = __shfl_up(incl, off);
-            if (lane >= off) incl += t;
-        }
-        if (i < n_tiles) out[i] = carry + incl - v;
-        carry += __shfl(incl, 63);
+    for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t t = __shfl_up(incl, off);
+        if (lane >= off) incl += t;
     }
-    if (lane == 0) totals[blockIdx.x] = carry;
+    uint32_t running = incl - sum;
+#pragma unroll 8
+    for (uint32_t i = from; i < to; ++i) {
+        out[i] = running;
+        running += row[i];
+    }
+    if (lane == 63) totals[blockIdx.x] = incl;
 }
 
 // Segment boundaries of the sorted assignment keys: offsets[c] = first position whose key is >= c
@@ -199,6 +203,24 @@ __global__ __launch_bounds__(256) void segment_sum_columns_kernel(
     }
 }
 
+// Stores a result that nothing on this compute die reads again at device scope ("sc1"): it is written through the
+// die's cache instead of staying there as a dirty line that the stream of point rows evicts later.  The k * d sums
+// are 1 % of an update's traffic, but written among the reads they cost 11 % of its time as ordinary stores and
+// 8 % written through (690, 665 and, with the stores left out, 615 us for a million rows of 4 KiB).
+__device__ __forceinline__ void store_through(float __attribute__((ext_vector_type(4)))* dst,
+                                              const float __attribute__((ext_vector_type(4))) v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_through(float __attribute__((ext_vector_type(2)))* dst,
+                                              const float __attribute__((ext_vector_type(2))) v) {
+    asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(dst), "v"(v) : "memory");
+}
+__device__ __forceinline__ void store_through(float __attribute__((ext_vector_type(1)))* dst,
+                                              const float __attribute__((ext_vector_type(1))) v) {
+    const float first = v[0];
+    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(dst), "v"(first) : "memory");
+}
+
 // Sums of the rows of every centroid's segment, in ascending point id (the reference's order of additions), so the
 // additions of one column are a chain and the time of a launch is the walk of the longest segment: hundreds of rows
 // with many centroids, tens of thousands in a mesoclustering.  One wavefront owns 64 * W consecutive columns of
@@ -265,7 +287,7 @@ __global__ __launch_bounds__(64) void segment_sum_deep_kernel(
         for (int u = 0; u < ROWS; ++u)
             if (j + u < j1) acc += ring[u];
     }
-    if (t < n_groups) reinterpret_cast<vec_t*>(sums + (size_t) c * d)[t] = acc;
+    if (t < n_groups) store_through(reinterpret_cast<vec_t*>(sums + (size_t) c * d) + t, acc);
 }
 
 __global__ __launch_bounds__(256) void scale_by_size_kernel(
