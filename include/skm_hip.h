@@ -188,6 +188,12 @@ int skm_shift(skm_ctx* ctx, const float* d_new, const float* d_prev, size_t k, s
  * out[j] = X[index[j]], norms_out[j] = norms_in[index[j]] (norm pointers may be NULL). */
 int skm_gather_rows(skm_ctx* ctx, const float* d_x, size_t d, const uint64_t* d_index, size_t m,
                     float* d_out, const float* d_norms_in, float* d_norms_out);
+/* The partitioned index HierarchicalSuperKMeans::Train builds between its mesoclustering and its fine clustering
+ * (hierarchical_superkmeans.h:270-286): d_out_ids lists the n points grouped by assignment, ascending inside each
+ * group, as 64-bit row ids for skm_gather_rows, and d_out_sizes[c] is the number of points assigned to c.  Runs the
+ * stable sort of skm_update on the device instead of a counting sort over a host copy of the assignments. */
+int skm_group_by_assignment(skm_ctx* ctx, const uint32_t* d_idx, size_t n, size_t k, uint64_t* d_out_ids,
+                            uint32_t* d_out_sizes);
 /* GetTrueAssignmentsFromIndirectionBuffer (hierarchical_superkmeans.h:763-779):
  * out[index[j]] = local[j] + offset. */
 int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_t* d_local, size_t m,

@@ -10,6 +10,7 @@
 #include <random>
 #include <stdexcept>
 #include <string>
+#include <vector>
 
 #include "skm_hip.h"
 
@@ -290,4 +291,53 @@ class Buffer {
 };
 
 } // namespace hip
+// The first k entries of {0, 1, ..., n - 1} after std::shuffle(first, last, rng), which is how the reference draws
+// its initial centroids (superkmeans.h:1100-1120: shuffle all n indices, keep k).  libstdc++'s shuffle for a
+// generator range below n * n is the forward walk "for i = 1 .. n-1: swap(a[i], a[uniform(0, i)])", each position
+// through one call of uniform_int_distribution<size_t> with the bounds as parameters.  Position i still holds i
+// when the walk reaches it and is never visited again afterwards, so what the first k positions end up with follows
+// from the draws alone: no n-entry array, no cache miss per swap (ten million indices take a third of the time).
+// Whether the library's shuffle is this walk is checked once per process on a fixed case; if it is not (another
+// standard library, or the two-positions-per-draw form libstdc++ uses for small n), the array is shuffled as before.
+class ShuffledPrefix {
+  public:
+    static std::vector<size_t> Draw(const size_t n, const size_t k, std::mt19937& rng) {
+        if (n >= MIN_N_FOR_WALK && k <= n && WalkMatches()) return ByWalk(n, k, rng);
+        return ByArray(n, k, rng);
+    }
+    static std::vector<size_t> ByArray(const size_t n, const size_t k, std::mt19937& rng) {
+        std::vector<size_t> all(n);
+        for (size_t i = 0; i < n; ++i) all[i] = i;
+        std::shuffle(all.begin(), all.end(), rng);
+        all.resize(std::min(k, n));
+        return all;
+    }
+    static std::vector<size_t> ByWalk(const size_t n, const size_t k, std::mt19937& rng) {
+        using distribution_t = std::uniform_int_distribution<size_t>;
+        using bounds_t = distribution_t::param_type;
+        distribution_t uniform;
+        const size_t head_n = std::min(k, n);
+        std::vector<size_t> head(head_n);
+        for (size_t i = 0; i < head_n; ++i) head[i] = i;
+        for (size_t i = 1; i < head_n; ++i) std::swap(head[i], head[uniform(rng, bounds_t(0, i))]);
+        for (size_t i = std::max<size_t>(head_n, 1); i < n; ++i) {
+            const size_t j = uniform(rng, bounds_t(0, i));
+            if (j < head_n) head[j] = i;  // position i held i; what it receives is never read again
+        }
+        return head;
+    }
+    // Below this many indices the array is cheap, and libstdc++ takes two positions from one draw while n * n fits
+    // the generator's range (n < 65,536).
+    static constexpr size_t MIN_N_FOR_WALK = size_t(1) << 17;
+    static bool WalkMatches() {
+        static const bool ok = [] {
+            const size_t n = MIN_N_FOR_WALK + 3;
+            std::mt19937 a(20240301u), b(20240301u);
+            if (ByArray(n, n, a) != ByWalk(n, n, b)) return false;
+            return a() == b();  // the same number of draws
+        }();
+        return ok;
+    }
+};
+
 } // namespace skmeans

@@ -114,6 +114,7 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         }
         const size_t total_samples = this->n_samples;
         this->AllocateState(n, k);
+        this->PrepareHostOutputs(total_samples);
         final_assignments.Reset(ctx, total_samples);
         final_centroids.Reset(ctx, k * d);
         this->partial_d = std::max<uint32_t>(MIN_PARTIAL_D, this->vertical_d / 2);
@@ -126,6 +127,13 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
             std::cout << "\n=== PHASE 1: MESOCLUSTERING (k=" << n_mesoclusters << " clusters) ===" << std::endl;
         // Rotation first: it runs on the device while the host draws the initial mesocluster centroids.
         const float* data_to_cluster = this->SampleAndRotateVectors(data, n, total_samples, rotate, on_device);
+        // The fine phase's helper objects (a device context each: a stream, pinned result slots) are made now, while
+        // the device rotates: their number depends on nothing the mesoclustering computes.
+        const size_t wanted = this->config.n_threads == 0 ? FINE_HELPERS_DEFAULT : this->config.n_threads;
+        const size_t n_helpers = std::max<size_t>(1, std::min<size_t>({wanted, FINE_HELPERS_MAX, n_mesoclusters}));
+        std::vector<std::unique_ptr<HierarchicalSuperKMeans>> helpers;
+        for (size_t h = 0; n_helpers > 1 && h < n_helpers; ++h)
+            helpers.emplace_back(new HierarchicalSuperKMeans(*this, FineHelperTag{}));
         this->GenerateCentroids(data, total_samples, n_mesoclusters, rotate, on_device);
         this->RotateOrCopy(this->horizontal_centroids.get(), this->prev_centroids.get(), n_mesoclusters, rotate);
         hip::Check(skm_norms(ctx, data_to_cluster, total_samples, d, d, this->data_norms.get()));
@@ -137,27 +145,24 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
                  hierarchical_config.use_blas_only, /*first_iteration_exact=*/true,
                  hierarchical_iteration_stats.mesoclustering_iteration_stats, hierarchical_config.early_termination);
 
-        // Assignments of the last search and the number of points they give every mesocluster.
-        // The reference takes the sizes from cluster_sizes, which SplitClusters has already edited when
-        // a mesocluster was empty in the last iteration (hierarchical_superkmeans.h:262-286); its
-        // partition of the points is then inconsistent with the assignments.  Here the sizes are
-        // recounted from the assignments, which is identical whenever no such split happened; an
-        // empty mesocluster simply receives no fine clusters.
-        mesoclusters_assignments.resize(total_samples);
-        this->d_assignments.Download(mesoclusters_assignments.data(), total_samples);
-        mesoclusters_sizes.assign(n_mesoclusters, 0u);
-        for (size_t i = 0; i < total_samples; ++i) mesoclusters_sizes[mesoclusters_assignments[i]]++;
-
-        // Point ids grouped by mesocluster, ascending inside each group (counting sort).
-        std::vector<uint64_t> indices_flat(total_samples);
+        // The number of points the last search gives every mesocluster, and the point ids grouped by mesocluster,
+        // ascending inside each group (hierarchical_superkmeans.h:262-286).  The reference takes the sizes from
+        // cluster_sizes, which SplitClusters has already edited when a mesocluster was empty in the last iteration;
+        // its partition of the points is then inconsistent with the assignments.  Here the sizes are recounted from
+        // the assignments, which is identical whenever no such split happened; an empty mesocluster simply receives
+        // no fine clusters.  Both come from one stable sort on the device: only the sizes travel to the host, and
+        // the assignments of the mesoclustering stay on the device (mesoclusters_assignments is left empty).
+        dbuf<uint64_t> d_indices(ctx, total_samples);
+        {
+            dbuf<uint32_t> d_meso_sizes(ctx, n_mesoclusters);
+            hip::Check(skm_group_by_assignment(ctx, this->d_assignments.get(), total_samples, n_mesoclusters, d_indices.get(),
+                                               d_meso_sizes.get()));
+            mesoclusters_sizes.assign(n_mesoclusters, 0u);
+            d_meso_sizes.Download(mesoclusters_sizes.data(), n_mesoclusters);
+        }
+        mesoclusters_assignments.clear();
         std::vector<size_t> offsets(n_mesoclusters + 1, 0);
         for (size_t m = 0; m < n_mesoclusters; ++m) offsets[m + 1] = offsets[m] + mesoclusters_sizes[m];
-        {
-            std::vector<size_t> cursor(offsets.begin(), offsets.end() - 1);
-            for (size_t i = 0; i < total_samples; ++i) indices_flat[cursor[mesoclusters_assignments[i]]++] = i;
-        }
-        dbuf<uint64_t> d_indices(ctx, total_samples);
-        d_indices.Upload(indices_flat.data(), total_samples);
 
         // ---- phase 2: fine clustering, one mesocluster after the other ----
         if (hierarchical_config.verbose)
@@ -186,18 +191,14 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         // counter.  Every problem is computed exactly as it would be alone; the statistics are put back in
         // mesocluster order afterwards.
         std::vector<std::vector<SuperKMeansIterationStats>> fine_stats(n_mesoclusters);
-        const size_t wanted = this->config.n_threads == 0 ? FINE_HELPERS_DEFAULT : this->config.n_threads;
-        const size_t n_helpers = std::max<size_t>(1, std::min<size_t>({wanted, FINE_HELPERS_MAX, n_mesoclusters}));
         hip::Check(skm_sync(ctx));  // everything the helpers read is complete
         if (n_helpers == 1) {
             dbuf<float> mesocluster_buffer(ctx, std::max<size_t>(1, max_mesocluster_size) * d);
             for (size_t m = 0; m < n_mesoclusters; ++m) FineClusterOne(in, m, mesocluster_buffer.get(), fine_stats[m]);
         } else {
-            std::vector<std::unique_ptr<HierarchicalSuperKMeans>> helpers;
             for (size_t h = 0; h < n_helpers; ++h) {
-                helpers.emplace_back(new HierarchicalSuperKMeans(*this, FineHelperTag{}));
-                helpers.back()->n_samples = std::max<size_t>(1, max_mesocluster_size);  // sizes the per-point buffers
-                helpers.back()->AllocateState(std::max<size_t>(1, max_mesocluster_size), std::max<size_t>(1, max_fineclusters));
+                helpers[h]->n_samples = std::max<size_t>(1, max_mesocluster_size);  // sizes the per-point buffers
+                helpers[h]->AllocateState(std::max<size_t>(1, max_mesocluster_size), std::max<size_t>(1, max_fineclusters));
             }
             std::atomic<size_t> next{0};
             std::vector<std::exception_ptr> failures(n_helpers);
@@ -247,8 +248,9 @@ class HierarchicalSuperKMeans : public SuperKMeans<q, alpha> {
         // (:484-499).  A point's norm is the same addend for all its distances, so assignments and centroids do
         // not depend on it, but the distances and therefore the refinement objectives the reference reports (and
         // its tests pin, tests/test_hierarchical_superkmeans.cpp:636-670) do.  The buffer is rebuilt here in the
-        // reference's order, whichever helper clustered which mesocluster.
-        for (size_t m = 0; m < n_mesoclusters; ++m) {
+        // reference's order, whichever helper clustered which mesocluster, when an exact refinement follows (nothing
+        // else reads it).
+        for (size_t m = 0; refinement_exact && hierarchical_config.iters_refinement > 0 && m < n_mesoclusters; ++m) {
             if (fine_clusters_nums[m] == 0 || mesoclusters_sizes[m] == 0) continue;
             hip::Check(skm_copy(ctx, this->data_norms.get(), fine_norms.get() + offsets[m],
                                 sizeof(float) * mesoclusters_sizes[m]));

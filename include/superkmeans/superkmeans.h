@@ -105,7 +105,7 @@ class SuperKMeans {
                   "only <f32, l2> is instantiated, as in the reference");
 
   public:
-    virtual ~SuperKMeans() = default;
+    virtual ~SuperKMeans() { FinishHostOutputs(); }
 
   protected:
     using centroid_value_t = skmeans_centroid_value_t<q>;
@@ -395,6 +395,7 @@ class SuperKMeans {
                 "Not enough samples to train. Try increasing the sampling_fraction or max_points_per_cluster");
         }
         AllocateState(n, n_clusters);
+        PrepareHostOutputs(n_samples);
         partial_d = std::max<uint32_t>(MIN_PARTIAL_D, vertical_d / 2);
         if (partial_d > vertical_d) partial_d = vertical_d;
         if (config.verbose) {
@@ -457,6 +458,7 @@ class SuperKMeans {
 
     // Device and host state sized like the reference's buffers (superkmeans.h:191-209).
     void AllocateState(const size_t n, const size_t k) {
+        FinishHostOutputs();  // a helper thread of an earlier, failed Train may still be touching the host buffers
         vertical_d = static_cast<uint32_t>(layout_t::GetDimensionSplit(d).vertical_d);
         centroids.Reset(ctx, k * d);
         horizontal_centroids.Reset(ctx, k * d);
@@ -756,9 +758,7 @@ class SuperKMeans {
             throw std::runtime_error("cannot draw more initial centroids than there are points");
         }
         std::mt19937 rng(config.seed);
-        std::vector<size_t> indices(n_points);
-        std::iota(indices.begin(), indices.end(), size_t{0});
-        std::shuffle(indices.begin(), indices.end(), rng);
+        const std::vector<size_t> indices = ShuffledPrefix::Draw(n_points, k, rng);
         if (on_device) {
             std::vector<uint64_t> rows(indices.begin(), indices.begin() + k);
             dbuf<uint64_t> d_rows(ctx, k);
@@ -850,14 +850,23 @@ class SuperKMeans {
     std::vector<centroid_value_t> GetOutputCentroids(bool should_unrotate) {
         // With a sink set the centroids go straight to the caller's buffer and the returned vector is empty.
         std::vector<centroid_value_t> out;
+        dbuf<float> unrotated;
+        if (should_unrotate) {
+            unrotated.Reset(ctx, n_clusters * d);
+            pruner->Unrotate(ctx, horizontal_centroids.get(), unrotated.get(), n_clusters);
+        }
+        FinishHostOutputs();
         centroid_value_t* dst = output_sink;
         if (dst == nullptr) {
-            out.resize(n_clusters * d);
+            if (prepared_centroids.size() == n_clusters * d) {
+                out = std::move(prepared_centroids);
+                prepared_centroids = std::vector<centroid_value_t>();
+            } else {
+                out.resize(n_clusters * d);
+            }
             dst = out.data();
         }
         if (should_unrotate) {
-            dbuf<float> unrotated(ctx, n_clusters * d);
-            pruner->Unrotate(ctx, horizontal_centroids.get(), unrotated.get(), n_clusters);
             unrotated.Download(dst, n_clusters * d);
         } else {
             horizontal_centroids.Download(dst, n_clusters * d);
@@ -962,10 +971,36 @@ class SuperKMeans {
 
     // Copies the device assignments / distances of the training points to the public host members.
     void PublishAssignments(const size_t count) {
+        FinishHostOutputs();
         d_assignments.Download(assignments.get(), count);
         host_distances.resize(count);
         distances.Download(host_distances.data(), count);
     }
+
+    // The host memory the end of Train fills: the assignments, the distances and the returned centroids.  Every
+    // fresh page costs a fault and a zeroing (20 ms for the 268 MB of 65,536 centroids of 1,024 dimensions), so a
+    // helper thread touches them while the device trains.  FinishHostOutputs comes before anything else reads or
+    // writes these buffers.
+    void PrepareHostOutputs(const size_t count) {
+        FinishHostOutputs();
+        const bool want_centroids = output_sink == nullptr;
+        const size_t bytes = count * (sizeof(uint32_t) + sizeof(float)) +
+                             (want_centroids ? n_clusters * d * sizeof(centroid_value_t) : 0);
+        if (bytes < HOST_OUTPUTS_AHEAD_BYTES) return;
+        host_outputs_thread = std::thread([this, count, want_centroids] {
+            try {
+                std::memset(assignments.get(), 0, count * sizeof(uint32_t));
+                host_distances.assign(count, 0.0f);
+                if (want_centroids) prepared_centroids.assign(n_clusters * d, centroid_value_t(0));
+            } catch (...) {
+                prepared_centroids.clear();  // the buffers are then made where they are filled
+            }
+        });
+    }
+    void FinishHostOutputs() {
+        if (host_outputs_thread.joinable()) host_outputs_thread.join();
+    }
+    static constexpr size_t HOST_OUTPUTS_AHEAD_BYTES = size_t(16) << 20;
 
     const size_t d;
     const size_t n_clusters;
@@ -1014,6 +1049,8 @@ class SuperKMeans {
     dbuf<float> rotated_queries, query_norms, gt_distances, recall_distances;
     dbuf<uint32_t> gt_assignments, promising_centroids;
     std::vector<float> host_distances;
+    std::vector<centroid_value_t> prepared_centroids;  // PrepareHostOutputs
+    std::thread host_outputs_thread;
     bool collect_prune_accounting = false;
     std::vector<std::vector<uint64_t>> prune_accounting;
 

@@ -53,6 +53,7 @@ _PROTOTYPES = {
          POINTER(c_uint64), POINTER(c_uint64)],
     ),
     "skm_update": (c_int, [c_void_p, _F, c_size_t, c_size_t, _F, c_size_t, _F, _F]),
+    "skm_group_by_assignment": (c_int, [c_void_p, _F, c_size_t, c_size_t, _F, _F]),
     "skm_scale_by_size": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t]),
     "skm_scale_by_size_fetch": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_uint32)]),
     "skm_normalize_rows": (c_int, [c_void_p, _F, c_size_t, c_size_t]),

@@ -453,20 +453,12 @@ int overflow_count_slot(skm_ctx* ctx, uint32_t** h_slot) {
     return SKM_OK;
 }
 
-} // namespace skm
-
-using namespace skm;
-
-extern "C" {
-
-int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_t* d_idx, size_t k,
-               float* d_out_sums, uint32_t* d_out_sizes) {
-    SKM_REQUIRE(ctx, "null context");
-    SKM_REQUIRE(d_out_sums && d_out_sizes, "null output");
-    SKM_REQUIRE(k > 0 && d > 0, "k and d must be positive");
-    SKM_REQUIRE(k < 0xffffffffULL && n < 0xffffffffULL, "n and k must fit in 32 bits");
-    SKM_REQUIRE(n == 0 || (d_x && d_idx), "null input");
-    ScopedStage st(ctx, "update_centroids");
+// Stable sort of the point ids by assignment (one radix pass per 7 or 8 key bits): *out_sorted_ids lists the n points
+// grouped by cluster, ascending inside each group, and (*out_offsets)[c] is the first position of cluster c
+// ((*out_offsets)[k] = n).  Both live in the context's workspace until its slots 1 and 4 are used again; the ids are
+// also kept as the context's visiting order of these n points.
+static int sort_by_assignment(skm_ctx* ctx, const uint32_t* d_idx, size_t n, size_t k, const uint32_t** out_sorted_ids,
+                              uint32_t** out_offsets) {
     // Scratch: keys/vals double buffers (4n u32), offsets (k+1), per-tile histograms.
     const int tile = n <= SORT_FEW_KEYS ? SORT_TILE_FEW_KEYS : SORT_TILE;
     const uint32_t n_tiles = (uint32_t) ((n + tile - 1) / tile);
@@ -533,6 +525,38 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         ctx->cluster_order_n = 0;
         SKM_TRY(skm_fill_u32(ctx, offsets, 0u, k + 1));
     }
+    *out_sorted_ids = sorted_ids;
+    *out_offsets = offsets;
+    return SKM_OK;
+}
+
+// Ids widened to the 64-bit row ids the gathers take, and the group sizes from the offsets.
+__global__ __launch_bounds__(256) void groups_out_kernel(
+    const uint32_t* __restrict__ sorted_ids, const uint32_t* __restrict__ offsets, size_t n, size_t k,
+    uint64_t* __restrict__ out_ids, uint32_t* __restrict__ out_sizes
+) {
+    const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out_ids[i] = sorted_ids[i];
+    if (i < k) out_sizes[i] = offsets[i + 1] - offsets[i];
+}
+
+} // namespace skm
+
+using namespace skm;
+
+extern "C" {
+
+int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_t* d_idx, size_t k,
+               float* d_out_sums, uint32_t* d_out_sizes) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(d_out_sums && d_out_sizes, "null output");
+    SKM_REQUIRE(k > 0 && d > 0, "k and d must be positive");
+    SKM_REQUIRE(k < 0xffffffffULL && n < 0xffffffffULL, "n and k must fit in 32 bits");
+    SKM_REQUIRE(n == 0 || (d_x && d_idx), "null input");
+    ScopedStage st(ctx, "update_centroids");
+    const uint32_t* sorted_ids = nullptr;
+    uint32_t* offsets = nullptr;
+    SKM_TRY(sort_by_assignment(ctx, d_idx, n, k, &sorted_ids, &offsets));
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(d_x) % 16 == 0) &&
                      (reinterpret_cast<uintptr_t>(d_out_sums) % 16 == 0);
     if (vec) {
@@ -552,6 +576,22 @@ int skm_update(skm_ctx* ctx, const float* d_x, size_t n, size_t d, const uint32_
         hipLaunchKernelGGL(segment_sum_columns_kernel, dim3((unsigned) k), dim3(256), 0, ctx->stream, d_x, d, sorted_ids, offsets, d_out_sums, d_out_sizes);
     }
     return check_hip(hipGetLastError(), "segment sum launch");
+}
+
+int skm_group_by_assignment(skm_ctx* ctx, const uint32_t* d_idx, size_t n, size_t k, uint64_t* d_out_ids,
+                            uint32_t* d_out_sizes) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(d_out_sizes, "null output");
+    SKM_REQUIRE(k > 0, "k must be positive");
+    SKM_REQUIRE(k < 0xffffffffULL && n < 0xffffffffULL, "n and k must fit in 32 bits");
+    SKM_REQUIRE(n == 0 || (d_idx && d_out_ids), "null argument");
+    const uint32_t* sorted_ids = nullptr;
+    uint32_t* offsets = nullptr;
+    SKM_TRY(sort_by_assignment(ctx, d_idx, n, k, &sorted_ids, &offsets));
+    const size_t threads = std::max(n, k);
+    hipLaunchKernelGGL(groups_out_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, ctx->stream, sorted_ids,
+                       offsets, n, k, d_out_ids, d_out_sizes);
+    return check_hip(hipGetLastError(), "groups_out_kernel launch");
 }
 
 int skm_scale_by_size(skm_ctx* ctx, float* d_sums, const uint32_t* d_sizes, size_t k, size_t d) {

@@ -47,6 +47,11 @@ struct skm_ctx {
     size_t h_ring_used = 0;
     void* h_pinned = nullptr;
     size_t h_pinned_bytes = 0;
+    // Lanes of a large download (skm_download of DOWNLOAD_LANES_MIN_BYTES or more into pageable memory): a stream
+    // and a pinned staging block each, made on first use.
+    static constexpr int DOWNLOAD_LANES = 4;
+    hipStream_t download_stream[DOWNLOAD_LANES] = {nullptr, nullptr, nullptr, nullptr};
+    void* download_staging = nullptr;  // DOWNLOAD_LANES blocks of DOWNLOAD_CHUNK bytes
     // Address, on this context's device, of the library's static scratch array (skm_assign_full_noalloc).
     void* noalloc_scratch = nullptr;
     bool prof = false;

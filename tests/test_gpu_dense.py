@@ -216,3 +216,18 @@ def test_upload_on_the_transfer_stream_orders_before_later_work(capi, ctx):
     assert np.allclose(out.download(), (X.astype(np.float64) ** 2).sum(1), rtol=1e-5)
     dX.free(), out.free()
 
+
+
+def test_large_download_through_the_lanes_is_byte_exact(capi, ctx):
+    """From 64 MiB a download goes through four threads, each moving every fourth 4 MiB chunk through its own pinned
+    block; the copy waits for the work queued before it.  Sizes with a ragged last chunk and with fewer chunks than
+    lanes' turns; the small path beside it.  Twice, so the second call reuses the lanes."""
+    g = np.random.default_rng(6)
+    for count in (16 * 1024 * 1024 + 12345, 16 * 1024 * 1024, 20_000_003, 1_000_001):
+        host = g.integers(0, 2 ** 32, count, dtype=np.uint32)
+        dev = ctx.array(host)
+        capi.check(ctx.lib.skm_fill_u32(ctx.handle, dev.ptr, 0xdeadbeef, 1000))  # queued work the copy must wait for
+        got = dev.download()
+        assert np.array_equal(got[:1000], np.full(1000, 0xdeadbeef, dtype=np.uint32))
+        assert np.array_equal(got[1000:], host[1000:])
+        dev.free()

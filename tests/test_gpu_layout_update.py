@@ -71,6 +71,25 @@ def test_update_sums_and_sizes_bit_exact(capi, ctx, oracle, n, d, k, nthreads):
         arr.free()
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,k", [(5000, 16), (100_000, 256), (300_001, 300), (1, 1), (70_000, 70_000), (2_000_000, 1000)])
+def test_group_by_assignment_is_the_counting_sort_of_the_reference(capi, ctx, n, k):
+    """The partitioned index between mesoclustering and fine clustering (reference hierarchical_superkmeans.h:270-286:
+    offsets from the sizes, then every point appended to its mesocluster's list in point order) equals a stable
+    argsort of the assignments; the sizes are the counts.  Integer work: array_equal."""
+    g = np.random.default_rng(n + k)
+    a = g.integers(0, k, n).astype(np.uint32)
+    if k > 3:
+        a[a == 1] = 0  # an empty group
+    dA, dI, dZ = ctx.array(a), ctx.empty(n, np.uint64), ctx.empty(k, np.uint32)
+    capi.check(ctx.lib.skm_group_by_assignment(ctx.handle, dA.ptr, n, k, dI.ptr, dZ.ptr))
+    ids, sizes = dI.download(), dZ.download()
+    assert np.array_equal(sizes, np.bincount(a, minlength=k).astype(np.uint32))
+    assert np.array_equal(ids, np.argsort(a, kind="stable").astype(np.uint64))
+    for arr in (dA, dI, dZ):
+        arr.free()
+
+
 def test_update_is_run_to_run_deterministic(capi, ctx):
     g = np.random.default_rng(0)
     X = g.standard_normal((50000, 96)).astype(np.float32)

@@ -45,6 +45,18 @@ def test_utils_header_matches_the_oracle_and_closed_forms(tmp_path, oracle):
     assert lines["timer_ok"] == "1"
 
 
+def test_shuffled_prefix_equals_std_shuffle(tmp_path):
+    """GenerateCentroids keeps the first k entries of std::shuffle over all n indices (reference superkmeans.h:1100-1120).
+    ShuffledPrefix derives them from the draws alone for large n; it must give the entries, and leave the generator in
+    the state, that shuffling the whole array gives: n on both sides of its size switch and of libstdc++'s own switch
+    at 65,536, k = 1, 5, n/3 and n, two seeds."""
+    exe = _build(tmp_path, "shuffled_prefix.cpp", "shuffled_prefix")
+    out = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "mismatches 0" in out.stdout
+    assert "equal 1" in out.stdout
+
+
 def test_reference_examples_compile_against_these_headers():
     """The reference's own example programs use nothing but the public headers: they must pass a syntax check
     against include/ unchanged.  Skipped where the reference checkout is absent."""
