@@ -267,6 +267,14 @@ int skm_ctx_create(int device, skm_ctx** out_ctx) {
         delete ctx;
         return check_hip(e, "hipStreamCreate");
     }
+    // The pinned block is made here rather than at its first use, which falls into the middle of an iteration:
+    // pinning host memory while kernels run holds them up (helper contexts are created while the device is idle).
+    const int rc = pinned_block(ctx);
+    if (rc != SKM_OK) {
+        (void) hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return rc;
+    }
     *out_ctx = ctx;
     return SKM_OK;
 }
