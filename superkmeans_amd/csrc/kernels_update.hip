@@ -351,6 +351,25 @@ constexpr int REDUCE_BLOCKS = 512;
 // Fixed-shape two-stage reductions in fp64 in one launch: block b sums elements b*256+tid, +512*256, ... and the
 // block that finishes last (a counter tells it) adds the 512 block sums in a fixed tree, so the association depends
 // only on the element count, never on which block came last.  The counter is left at zero for the next launch.
+// Sum of one double per thread of a 256-thread workgroup in the tree s[t] += s[t + off], off = 128, 64, ..., 1
+// (thread 0 holds the result).  The levels off = 128 and 64 pair values of different wavefronts and go through LDS;
+// from off = 32 down both operands sit in wavefront 0, where lane t takes lane t + off's value with a shuffle: the
+// same additions in the same order with three barriers instead of nine.
+__device__ __forceinline__ double block_tree_sum(const double mine, double* s) {
+    s[threadIdx.x] = mine;
+    __syncthreads();
+    if (threadIdx.x < 128) s[threadIdx.x] += s[threadIdx.x + 128];
+    __syncthreads();
+    double v = 0.0;
+    if (threadIdx.x < 64) {
+        v = s[threadIdx.x] + s[threadIdx.x + 64];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off);  // lanes at or above off compute values nobody reads
+    }
+    __syncthreads();  // s may be written again by the caller
+    return v;
+}
+
 template <int MODE>  // 0: sum a[i]; 1: sum (a[i]-b[i])^2; 2: sum of uint32 a[i] (as exact integers)
 __global__ __launch_bounds__(256) void reduce_kernel(
     const float* __restrict__ a, const float* __restrict__ b, size_t n, double* __restrict__ partial,
@@ -370,14 +389,9 @@ __global__ __launch_bounds__(256) void reduce_kernel(
             acc += (double) reinterpret_cast<const uint32_t*>(a)[i];
         }
     }
-    s[threadIdx.x] = acc;
-    __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
-        __syncthreads();
-    }
+    const double block_sum = block_tree_sum(acc, s);
     if (threadIdx.x == 0) {
-        partial[blockIdx.x] = s[0];
+        partial[blockIdx.x] = block_sum;
         __threadfence();  // the block sum is visible device-wide before the counter says so
         s_done = atomicAdd(counter, 1u);
     }
@@ -385,14 +399,9 @@ __global__ __launch_bounds__(256) void reduce_kernel(
     if (s_done != REDUCE_BLOCKS - 1) return;
     __threadfence();
     const volatile double* all = partial;  // written by other compute units: read past this one's cache
-    s[threadIdx.x] = all[threadIdx.x] + all[threadIdx.x + 256];
-    __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if (threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
-        __syncthreads();
-    }
+    const double total = block_tree_sum(all[threadIdx.x] + all[threadIdx.x + 256], s);
     if (threadIdx.x == 0) {
-        out[0] = s[0];
+        out[0] = total;
         *counter = 0u;
         if (word_in) *word_out = *word_in;  // a device word the host wants with the same wait (earlier kernels wrote it)
     }
