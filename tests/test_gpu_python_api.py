@@ -129,3 +129,21 @@ def test_train_with_queries(pkg):  # python/tests/test_superkmeans.py:49-64 of t
     assert any(s.recall > 0.0 for s in km.iteration_stats)
     with pytest.raises(ValueError, match="dimensionality"):
         pkg.SuperKMeans(n_clusters=k, dimensionality=d).train(data, queries=queries[:, :100].copy())
+
+
+def test_returned_centroids_prepared_ahead_equal_the_plain_path(pkg, capi):
+    """From 16 MiB of host results Train touches the vector it returns (and the assignment and distance buffers) on a
+    helper thread while the device works; the C ABI's train writes into the caller's buffer instead and starts no
+    such thread for the centroids.  Same seed, same data: the two must return the same bits, the object must
+    refuse a second Train, and its destructor must find the thread joined."""
+    n, d, k = 9000, 1024, 4200  # 4200 x 1024 floats = 17.2 MB
+    data = _data(n, d, seed=9)
+    km = pkg.SuperKMeans(n_clusters=k, dimensionality=d, iters=2, sampling_fraction=1.0, seed=5)
+    got = km.train(data)
+    ck = capi.KMeans(k, d, iters=2, sampling_fraction=1.0, seed=5)
+    want = ck.train(data)
+    ck.close()
+    assert got.shape == (k, d) and np.array_equal(got, want)
+    with pytest.raises(RuntimeError, match="already been trained"):
+        km.train(data)
+    del km
