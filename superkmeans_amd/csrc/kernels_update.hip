@@ -346,11 +346,19 @@ __global__ __launch_bounds__(256) void edit_rows_kernel(float* __restrict__ c, s
     }
 }
 
+// Workgroups of a reduction: one per 2,048 elements, at most 512.  A short input (the distances of a fine-phase
+// problem, the centroids of a small one) would otherwise pay for 512 workgroups that hold one element per thread
+// or none, and above all for their 512 additions to one counter, which the memory system performs one after the other.
 constexpr int REDUCE_BLOCKS = 512;
+constexpr size_t REDUCE_ELEMENTS_PER_BLOCK = 2048;
+static inline unsigned reduce_blocks(const size_t n) {
+    const size_t wanted = (n + REDUCE_ELEMENTS_PER_BLOCK - 1) / REDUCE_ELEMENTS_PER_BLOCK;
+    return (unsigned) std::min<size_t>(REDUCE_BLOCKS, std::max<size_t>(1, wanted));
+}
 
-// Fixed-shape two-stage reductions in fp64 in one launch: block b sums elements b*256+tid, +512*256, ... and the
-// block that finishes last (a counter tells it) adds the 512 block sums in a fixed tree, so the association depends
-// only on the element count, never on which block came last.  The counter is left at zero for the next launch.
+// Fixed-shape two-stage reductions in fp64 in one launch: block b of B sums elements b*256+tid, +B*256, ... and the
+// block that finishes last (a counter tells it) adds the B <= 512 block sums in a fixed tree, so the association
+// depends only on the element count, never on which block came last.  The counter is left at zero for the next launch.
 // Sum of one double per thread of a 256-thread workgroup in the tree s[t] += s[t + off], off = 128, 64, ..., 1
 // (thread 0 holds the result).  The levels off = 128 and 64 pair values of different wavefronts and go through LDS;
 // from off = 32 down both operands sit in wavefront 0, where lane t takes lane t + off's value with a shuffle: the
@@ -379,16 +387,25 @@ __global__ __launch_bounds__(256) void reduce_kernel(
     __shared__ double s[256];
     __shared__ uint32_t s_done;
     double acc = 0.0;
-    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t) REDUCE_BLOCKS * 256) {
-        if (MODE == 0) {
-            acc += (double) a[i];
-        } else if (MODE == 1) {
+    const auto term = [&](const size_t i) -> double {
+        if (MODE == 0) return (double) a[i];
+        if (MODE == 1) {
             const float t = a[i] - b[i];
-            acc += (double) (t * t);
-        } else {
-            acc += (double) reinterpret_cast<const uint32_t*>(a)[i];
+            return (double) (t * t);
         }
+        return (double) reinterpret_cast<const uint32_t*>(a)[i];
+    };
+    // the elements of a thread, in ascending order; four at a time are requested before any is added
+    const size_t stride = (size_t) gridDim.x * 256;
+    size_t i = (size_t) blockIdx.x * 256 + threadIdx.x;
+    for (; i + 3 * stride < n; i += 4 * stride) {
+        const double t0 = term(i), t1 = term(i + stride), t2 = term(i + 2 * stride), t3 = term(i + 3 * stride);
+        acc += t0;
+        acc += t1;
+        acc += t2;
+        acc += t3;
     }
+    for (; i < n; i += stride) acc += term(i);
     const double block_sum = block_tree_sum(acc, s);
     if (threadIdx.x == 0) {
         partial[blockIdx.x] = block_sum;
@@ -396,10 +413,13 @@ __global__ __launch_bounds__(256) void reduce_kernel(
         s_done = atomicAdd(counter, 1u);
     }
     __syncthreads();
-    if (s_done != REDUCE_BLOCKS - 1) return;
+    if (s_done != gridDim.x - 1) return;
     __threadfence();
     const volatile double* all = partial;  // written by other compute units: read past this one's cache
-    const double total = block_tree_sum(all[threadIdx.x] + all[threadIdx.x + 256], s);
+    // sums of blocks that do not exist count as zero: with 512 blocks this is the sum it always was
+    const double low = threadIdx.x < gridDim.x ? all[threadIdx.x] : 0.0;
+    const double high = threadIdx.x + 256 < gridDim.x ? all[threadIdx.x + 256] : 0.0;
+    const double total = block_tree_sum(low + high, s);
     if (threadIdx.x == 0) {
         out[0] = total;
         *counter = 0u;
@@ -428,11 +448,11 @@ static int reduce_enqueue(skm_ctx* ctx, int mode, const float* a, const float* b
     uint32_t* counter = nullptr;
     SKM_TRY(reduction_counter(ctx, &counter));
     if (mode == 0)
-        hipLaunchKernelGGL(reduce_kernel<0>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
+        hipLaunchKernelGGL(reduce_kernel<0>, dim3(reduce_blocks(n)), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     else if (mode == 1)
-        hipLaunchKernelGGL(reduce_kernel<1>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
+        hipLaunchKernelGGL(reduce_kernel<1>, dim3(reduce_blocks(n)), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     else
-        hipLaunchKernelGGL(reduce_kernel<2>, dim3(REDUCE_BLOCKS), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
+        hipLaunchKernelGGL(reduce_kernel<2>, dim3(reduce_blocks(n)), dim3(256), 0, ctx->stream, a, b, n, partial, counter, h_slot, d_word, h_word);
     return check_hip(hipGetLastError(), "reduce_kernel launch");
 }
 
