@@ -44,13 +44,13 @@ PEAK_HBM_GBPS = 8000.0
 # not profiled.  They describe the build the summaries were taken with; a change to a kernel needs a new profile run.
 #   profiles/gemm_argmin_kernel_assign_n1M_d1024_k10k_hbm_traffic.md: the two gemm_argmin_kernel launches of an Assign pass
 MEASURED_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000): int(((31_551_641 + 2_005_720) * 1.943 + 609_375 + 7_812) * 1024),
+    (1_000_000, 1024, 10_000): int(((31_605_895 + 2_005_959) * 1.943 + 609_375 + 7_812) * 1024),
 }
 #   same file: every seed_distance_kernel, prune_list_kernel and prune_kernel launch of one Train of (n, d, k, iterations)
 MEASURED_PRUNE_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000, 10): int((48_503_002 * 1.943 + 1_477_284) * 1024),
+    (1_000_000, 1024, 10_000, 10): int((48_587_738 * 1.943 + 1_477_281) * 1024),
     # profiles/train_n2M_d1536_k4096_kernel_stats_list_walk_traffic.md
-    (2_000_000, 1536, 4_096, 10): int((843_824_206 * 1.943 + 2_897_306) * 1024),
+    (2_000_000, 1536, 4_096, 10): int((843_855_099 * 1.943 + 2_897_329) * 1024),
 }
 
 
