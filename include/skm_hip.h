@@ -56,20 +56,38 @@ int skm_sync(skm_ctx* ctx);
 int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
 
 /* Which kernel computes the partial distances of skm_assign_pruned (tuning and test knob; results do not depend on
- * it): 0 = automatic (default: the register-stationary kernel for partial_d <= 160 and at least 131,072 points per
+ * it): 0 = automatic (default: the register-stationary kernel for partial_d <= 160 and at least 49,152 points per
  * call, the tiled 128 x 128 kernel otherwise), 1 = always the tiled kernel, 2 = the register-stationary kernel
  * whenever partial_d <= 160 and the rows are 16-byte aligned, whatever the number of points. */
 int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which);
 
+/* Which kernel walks the candidate lists of skm_assign_pruned (tuning and test knob; results do not depend on it):
+ * 0 = automatic (default: eight points pooled per wavefront for calls of at least 32,768 points whose rows are 16-byte
+ * aligned with d a multiple of 4, except for the second pass over points whose lists overflowed; one point per
+ * wavefront otherwise), 1 = always one point per wavefront, 2 = pooled wherever the rows allow it. */
+int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which);
+/* Into how many launches the pooled walk of a call is split, each over a contiguous range of the batches of 1024
+ * centroids, all points walking one range before any walks the next (default 1; capped at the number of batches;
+ * results do not depend on it).  With one launch per batch the compute dies gather from one batch's blocks at a time
+ * and less than half as many gathers miss their L2, but the launches' tails and the reloaded per-point state cost
+ * more time than the misses did, which the memory-side cache serves: a knob for measuring that trade. */
+int skm_ctx_set_walk_launches(skm_ctx* ctx, int launches);
+
 /* Device memory and transfers (stand in for the reference's std::unique_ptr<float[]> buffers,
  * superkmeans.h:191-201). */
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr);
+/* Waits for this context's streams, then hands the block to the per-device cache below, from which the next allocation
+ * of about its size, by any context of the process, may take it at once.  No other context and no other stream may
+ * still have work queued that uses the block when it is freed. */
 int skm_free(skm_ctx* ctx, void* d_ptr);
 /* Blocks released through skm_free, by a context's workspace or by skm_ctx_destroy are kept per device and handed
  * out again by later allocations of about the same size (allocating and releasing the multi-gigabyte buffers of a
- * Train costs milliseconds each time, and a release waits for the whole device).  The cache holds at most 96 GiB or
- * 2,048 blocks, empties itself when an allocation fails, and is emptied on request by this call. */
-int skm_device_cache_trim(int device);
+ * Train costs milliseconds each time, and a release waits for the whole device).  The cache holds at most 48 GiB
+ * (or the number of bytes in SKM_DEVICE_CACHE_BYTES when the process first uses the device; 0 keeps nothing) and
+ * 2,048 blocks, and empties itself when an allocation of this process fails.  Other processes on the same GPU do not
+ * see these blocks as free: lower the limit, or trim, where the GPU is shared. */
+int skm_device_cache_set_limit(int device, size_t bytes); /* blocks beyond the new limit go back to the driver */
+int skm_device_cache_trim(int device);                    /* returns every idle block to the driver */
 int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);
 /* Upload on the context's transfer stream: work queued on the context before the call keeps running during the

@@ -27,9 +27,12 @@ _PROTOTYPES = {
     "skm_sync": (c_int, [c_void_p]),
     "skm_ctx_set_workspace_limit": (c_int, [c_void_p, c_size_t]),
     "skm_ctx_set_candidate_kernel": (c_int, [c_void_p, c_int]),
+    "skm_ctx_set_walk_kernel": (c_int, [c_void_p, c_int]),
+    "skm_ctx_set_walk_launches": (c_int, [c_void_p, c_int]),
     "skm_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "skm_free": (c_int, [c_void_p, c_void_p]),
     "skm_device_cache_trim": (c_int, [c_int]),
+    "skm_device_cache_set_limit": (c_int, [c_int, c_size_t]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_upload_overlapped": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_householder_q": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -276,7 +276,7 @@ __global__ __launch_bounds__(512 / FM, FM) void gemm_candidates_stationary_kerne
 
     // ---- sweep: step t publishes tile t + 1, tests tile t - 1, requests tile t + 2 and multiplies tile t ----
     // The appends of a step are issued before its loads, so waiting for those loads a step later never waits
-    // for stores.  Step 0 tests nothing (no column is live yet); the last step multiplies a tile past the end (zeros).
+    // for stores.  Step 0 tests nothing; the last step multiplies a tile past the end (zeros).
     const int tiles = (M + CS_TN - 1) / CS_TN;
     request(0);
     publish(0);
@@ -285,7 +285,7 @@ __global__ __launch_bounds__(512 / FM, FM) void gemm_candidates_stationary_kerne
     fetch(0, 0, fb0, fb1);
     for (int t = 0; t <= tiles; ++t) {
         publish((t + 1) & 1);
-        emit(t - 1);
+        if (t > 0) emit(t - 1);
         request(t + 2);
         request_norms(t);
         __builtin_amdgcn_sched_barrier(0);
@@ -301,8 +301,10 @@ __global__ __launch_bounds__(512 / FM, FM) void gemm_candidates_stationary_kerne
 }
 
 // Up to 11 groups of 8 columns a wavefront holds the fragments of 64 points next to its 64 x 64 accumulators
-// (2 wavefronts per SIMD, 256 registers each) and two workgroups of 4 wavefronts share a CU; from 12 to 20 groups
-// it holds 32 points, and one workgroup of 8 wavefronts has the CU's LDS to itself.
+// (256 registers) and up to 10 groups two such workgroups of 4 wavefronts share a CU (79,872 bytes of LDS each; at 11
+// groups 83,968 bytes, so one workgroup has the CU to itself: measured at d' = 83 and 88 that is as fast as, or 2 %
+// faster than, the 8-wavefront shape); from 12 to 20 groups a wavefront holds 32 points and one workgroup of 8
+// wavefronts has the CU's LDS to itself.
 constexpr int CS_MAX_GROUPS_WIDE = 11;
 constexpr int CS_MAX_GROUPS = 20;
 

@@ -1,117 +1,23 @@
-// Pruned top-1 search: one wavefront per point walks the batches of 1024 centroids in order and
-// reproduces PDXearch::Top1PartialSearchWithThresholdAndPartialDistances / Prune / SetBestCandidate
+// Pruned top-1 search over per-point candidate lists, one wavefront per point: walks the batches of 1024 centroids
+// in order and reproduces PDXearch::Top1PartialSearchWithThresholdAndPartialDistances / Prune / SetBestCandidate
 // (reference pdx/pdxearch.h:118-238,266-327) and the per-row body of
-// BatchComputer::FindNearestNeighborWithPruning (distance_computers/batch_computers.h:357-405).
+// BatchComputer::FindNearestNeighborWithPruning (distance_computers/batch_computers.h:357-405).  Also the seed
+// distances of the search.  This walk serves rows that are not 16-byte aligned; kernels_prune_pool.hip holds the walk
+// with several points per wavefront that serves all others.
 //
 // Wavefront mapping
-//   * first test against best * ratios[d'] : 64 partial distances per step, survivors compacted in
-//     ascending position order with a ballot + prefix popcount into an LDS list
-//     (InitPositionsArray, scalar_computers.h:87-98);
-//   * every 64-dimension horizontal block: 4 survivors per step, 16 lanes x float4 each, reduced
-//     with four cross-lane exchanges, followed by the same ballot compaction
+//   * first test against best * ratios[d']: the candidates of the batch, 64 per step, survivors compacted with a
+//     ballot + prefix popcount into an LDS list (InitPositionsArray, scalar_computers.h:87-98);
+//   * every 64-dimension horizontal block: 32 survivors per pass, 16 lanes x float4 each, reduced with four
+//     cross-lane exchanges, followed by the same ballot compaction
 //     (EvaluatePruningPredicateOnPositionsArray, pdxearch.h:67-80);
 //   * the [d', vertical_d) dimensions are read last from the dense auxiliary copy;
 //   * survivors of the final test (ratio 1) update the best candidate, lowest position first.
 // The threshold of a batch is fixed while the batch is processed and only tightens between
 // batches, exactly as on the CPU, so the order in which survivors are visited cannot change results.
-#include "skm_internal.h"
-
-#include <float.h>
+#include "prune_common.h"
 
 namespace skm {
-
-constexpr int PRUNE_WAVES = 4;
-constexpr int PRUNE_CAP = SKM_Y_BATCH_SIZE;
-constexpr int LIST_PAD = 32;  // survivors per pass of the list walk
-
-struct PruneArgs {
-    const float* partial;  // n_chunk x ld_partial partial distances over the first partial_d dims
-    int64_t ld_partial;
-    const float* x;        // n_chunk x d rotated points
-    const float* c;        // k x d row-major centroids
-    const float* pdx;      // PDX copy of c
-    const float* aux;      // k x vertical_d
-    const float* ratios;   // d + 1
-    uint32_t* idx;         // in: previous assignment, out: new assignment
-    float* dist;           // out
-    uint32_t* not_pruned;  // out: per-point count of survivors of the first test, summed over batches
-    unsigned long long* stage_pairs;  // optional accounting, may be null
-    int n, k, d, vertical_d, partial_d;
-};
-
-// Sum over each group of 16 consecutive lanes, returned in all of them.  Rotations inside a row of 16 lanes are
-// data-parallel primitives of the vector unit (no trip through the LDS crossbar); the pairing is that of a
-// butterfly over lane distances 8, 4, 2, 1, so every lane adds the same pairs in the same order.
-template <int N>
-__device__ __forceinline__ float row_ror(float v) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x120 + N, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float group16_sum(float v) {
-    v += row_ror<8>(v);
-    v += row_ror<4>(v);
-    v += row_ror<2>(v);
-    v += row_ror<1>(v);
-    return v;
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
-}
-
-// Which point a wavefront takes.  Workgroups go to the eight compute dies in turn (workgroup b runs on die b % 8, each
-// with its own L2), so the grid is read as eight contiguous ranges of slots, one per die: consecutive slots, which
-// under a cluster order hold points that gather the same centroid rows and blocks, stay on one die.  The launch has
-// 8 * ceil(workgroups / 8) workgroups; a slot past the end returns -1.
-__device__ __forceinline__ int point_of_wave(const uint32_t* __restrict__ order, int n, int waves_per_group) {
-    const int per_die = (int) (gridDim.x / 8);
-    const int group = (int) (blockIdx.x % 8) * per_die + (int) (blockIdx.x / 8);
-    const int slot = group * waves_per_group + (int) (threadIdx.x >> 6);
-    if (slot >= n) return -1;
-    return order ? (int) order[slot] : slot;
-}
-inline unsigned die_striped_groups(int n, int waves_per_group) {
-    const unsigned groups = (unsigned) ((n + waves_per_group - 1) / waves_per_group);
-    return (groups + 7) / 8 * 8;
-}
-
-// The same pointer, said to be equal in all lanes (it is: it derives from the batch and block indices) and to point to
-// global memory (an address built from integers is otherwise taken for a flat one, whose loads are waited for all at
-// once): the compiler then keeps it in scalar registers and a gather needs only its 32-bit lane offset in a vector
-// register.
-typedef const char __attribute__((address_space(1)))* global_bytes_t;
-typedef float gather4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ global_bytes_t uniform_pointer(const void* p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t) v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t) (v >> 32));
-    return reinterpret_cast<global_bytes_t>(((uint64_t) hi << 32) | lo);
-}
-// Four floats at byte offset `off` of a block (16-byte load when VEC).
-template <bool VEC>
-__device__ __forceinline__ float4 gather4(global_bytes_t base, uint32_t off) {
-    if (VEC) {
-        const gather4_t g = *reinterpret_cast<const gather4_t __attribute__((address_space(1)))*>(base + off);
-        return make_float4(g.x, g.y, g.z, g.w);
-    }
-    const float __attribute__((address_space(1)))* f = reinterpret_cast<const float __attribute__((address_space(1)))*>(base + off);
-    return make_float4(f[0], f[1], f[2], f[3]);
-}
-
-// Four consecutive floats of a point row (16-byte load when rows are aligned).
-template <bool VEC>
-__device__ __forceinline__ float4 load_x4(const float* p) {
-    if (VEC) return *reinterpret_cast<const float4*>(p);
-    return make_float4(p[0], p[1], p[2], p[3]);
-}
-
-// The same for data that is read once per launch: a non-temporal load, which leaves the caches to the centroids.
-__device__ __forceinline__ float4 load_once4(const float* p) {
-    typedef float v4f __attribute__((ext_vector_type(4)));
-    const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f*>(p));
-    return make_float4(v.x, v.y, v.z, v.w);
-}
 
 // Keeps the survivors whose accumulated distance is below thr, preserving order. In-place: slot s
 // is rewritten only by elements read from slots >= s, and each step reads before it writes.
@@ -132,190 +38,6 @@ __device__ __forceinline__ int compact_survivors(uint16_t* pos, float* acc, int 
         out += __popcll(mask);
     }
     return out;
-}
-
-template <bool VEC>
-__global__ __launch_bounds__(PRUNE_WAVES * 64) void prune_kernel(PruneArgs a) {
-    __shared__ uint16_t s_pos[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];  // padded as in prune_list_kernel
-    __shared__ float s_acc[PRUNE_WAVES][PRUNE_CAP + LIST_PAD];
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    const int p = point_of_wave(nullptr, a.n, PRUNE_WAVES);  // consecutive rows stay on one compute die
-    if (p < 0) return;
-    uint16_t* pos = s_pos[wave];
-    float* acc = s_acc[wave];
-    const int d = a.d, V = a.vertical_d, dp = a.partial_d;
-    const int H = d - V;
-    const int n_hblocks = H / SKM_H_DIM_SIZE;
-    // Accounting counters come in SKM_ACCT_COPIES striped copies (summed by the host) so that the
-    // atomics of concurrently running workgroups spread over many addresses.
-    unsigned long long* acct = a.stage_pairs ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
-    const float* xq = a.x + (int64_t) p * d;
-    const int sub = lane & 15;   // lane within a 16-lane group
-    const int grp = lane >> 4;   // which of the 4 survivors handled per step
-
-    // Distance to the previous assignment over all d dimensions (batch_computers.h:372-377).
-    uint32_t best_idx = a.idx[p];
-    float best;
-    {
-        const float* cp = a.c + (int64_t) best_idx * d;
-        float s = 0.0f;
-        if (VEC) {
-            for (int t = lane * 4; t < d; t += 256) {
-                const float4 xv = *reinterpret_cast<const float4*>(xq + t);
-                const float4 cv = *reinterpret_cast<const float4*>(cp + t);
-                float e;
-                e = cv.x - xv.x; s += e * e;
-                e = cv.y - xv.y; s += e * e;
-                e = cv.z - xv.z; s += e * e;
-                e = cv.w - xv.w; s += e * e;
-            }
-        } else {
-            for (int t = lane; t < d; t += 64) {
-                const float e = cp[t] - xq[t];
-                s += e * e;
-            }
-        }
-        best = wave_sum(s);
-    }
-
-    uint32_t not_pruned_total = 0;
-    const int n_batches = (a.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE;
-    const float* prow = a.partial + (int64_t) p * a.ld_partial;
-    for (int jb = 0; jb < n_batches; ++jb) {
-        const int base = jb * SKM_Y_BATCH_SIZE;
-        const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
-        const uint32_t prev_top_1 = best_idx;
-        // ---- first test on the GEMM partial distances ----
-        float thr = best * a.ratios[dp];
-        int cnt = 0;
-        for (int c0 = 0; c0 < m; c0 += 64) {
-            const int c = c0 + lane;
-            const bool in = c < m;
-            const float v = in ? prow[base + c] : 0.0f;
-            const bool keep = in && (v < thr);
-            const unsigned long long mask = __ballot(keep);
-            if (keep) {
-                const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
-                pos[slot] = (uint16_t) c;
-                acc[slot] = v;
-            }
-            cnt += __popcll(mask);
-        }
-        not_pruned_total += (uint32_t) cnt;
-        if (acct && lane == 0 && cnt) atomicAdd(&acct[0], (unsigned long long) cnt);
-        // Only survivor is the incumbent: nothing to do (pdxearch.h:140-143).
-        if (cnt == 1 && (uint32_t) (base + pos[0]) == prev_top_1) continue;
-        if (cnt == 0) continue;
-
-        // ---- horizontal blocks of 64 dimensions, PDX layout (pdxearch.h:149-180) ----
-        const float* chunk = a.pdx + (int64_t) base * d;
-        int dims_seen = dp;
-        float4 xv_next = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        if (n_hblocks > 0) xv_next = load_x4<VEC>(xq + V + sub * 4);
-        for (int hb = 0; hb < n_hblocks && cnt > 0; ++hb) {
-            if (acct && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
-            const float* blk = chunk + (int64_t) V * m + (int64_t) hb * m * SKM_H_DIM_SIZE;
-            // This block's slice of the point was requested one block ago; the next one is requested now.
-            const float4 xv = xv_next;
-            if (hb + 1 < n_hblocks) xv_next = load_x4<VEC>(xq + V + (hb + 1) * SKM_H_DIM_SIZE + sub * 4);
-            // 32 survivors per pass: the eight gathers of a lane are issued before any of them is used.  Slots past
-            // the last survivor read the pad (position 0) and their sums land in the pad.
-            if (lane < LIST_PAD) pos[cnt + lane] = 0;
-            const global_bytes_t blk_bytes = uniform_pointer(blk);
-            const uint32_t lane_bytes = (uint32_t) sub * 16u;
-            for (int s0 = 0; s0 < cnt; s0 += 32) {
-                float4 cv[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const uint32_t cpos = pos[s0 + 4 * u + grp];
-                    cv[u] = gather4<VEC>(blk_bytes, (cpos << 8) | lane_bytes);
-                }
-                float mine = 0.0f;
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    float e, part = 0.0f;
-                    e = xv.x - cv[u].x; part += e * e;
-                    e = xv.y - cv[u].y; part += e * e;
-                    e = xv.z - cv[u].z; part += e * e;
-                    e = xv.w - cv[u].w; part += e * e;
-                    part = group16_sum(part);
-                    mine = sub == u ? part : mine;
-                }
-                if (sub < 8) acc[s0 + 4 * sub + grp] += mine;
-            }
-            dims_seen += SKM_H_DIM_SIZE;
-            thr = best * a.ratios[dims_seen];
-            cnt = compact_survivors(pos, acc, cnt, thr, lane);
-            // Only the incumbent is left: the best candidate stays what it is whatever the remaining steps do
-            // (pdxearch.h:140-143 applied after a step); with per-step accounting it keeps walking.
-            if (cnt == 1 && acct == nullptr && (uint32_t) (base + pos[0]) == prev_top_1) cnt = 0;
-        }
-
-        // ---- remaining vertical dimensions [d', V) from the dense auxiliary copy (pdxearch.h:183-216) ----
-        if (cnt > 0 && dp < V) {
-            if (acct && lane == 0) atomicAdd(&acct[1 + n_hblocks], (unsigned long long) cnt);
-            const int left = V - dp;
-            for (int s0 = 0; s0 < cnt; s0 += 4) {
-                const int s = s0 + grp;
-                const bool in = s < cnt;
-                const int cpos = in ? pos[s] : pos[0];
-                const float* cb = a.aux + (int64_t) (base + cpos) * V + dp;
-                // Four independent loads per operand in flight; the sum keeps the order t = sub, sub + 16, ...
-                float part = 0.0f;
-                for (int t = sub; t < left; t += 64) {
-                    float xe[4], ce[4];
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const int tt = t + 16 * u;
-                        xe[u] = tt < left ? xq[dp + tt] : 0.0f;
-                        ce[u] = tt < left ? cb[tt] : 0.0f;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; ++u) {
-                        const float e = xe[u] - ce[u];
-                        part += e * e;
-                    }
-                }
-                part = group16_sum(part);
-                if (in && sub == 0) acc[s] += part;
-            }
-            thr = best * a.ratios[d];
-            cnt = compact_survivors(pos, acc, cnt, thr, lane);
-        }
-
-        // ---- SetBestCandidate (pdxearch.h:223-238): strict <, lowest position wins ties ----
-        if (cnt > 0) {
-            float bv = FLT_MAX;
-            int bp = 0x7fffffff;
-            for (int s = lane; s < cnt; s += 64) {
-                const float v = acc[s];
-                const int q = pos[s];
-                if (v < bv || (v == bv && q < bp)) {
-                    bv = v;
-                    bp = q;
-                }
-            }
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                const float ov = __shfl_xor(bv, off);
-                const int op = __shfl_xor(bp, off);
-                if (ov < bv || (ov == bv && op < bp)) {
-                    bv = ov;
-                    bp = op;
-                }
-            }
-            if (bp != 0x7fffffff && bv < best) {
-                best = bv;
-                best_idx = (uint32_t) (base + bp);
-            }
-        }
-    }
-    if (lane == 0) {
-        a.idx[p] = best_idx;
-        a.dist[p] = best;
-        a.not_pruned[p] = not_pruned_total;
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -378,33 +100,13 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
 }
 
 // ---------------------------------------------------------------------------------------------
-// Pruned search over per-point candidate lists (see gemm_candidates_kernel).  Identical to
-// prune_kernel except for the first test of a batch, which filters the point's candidates that
-// belong to the batch with the exact threshold best * ratios[d'] instead of scanning 1024 dense
-// partial distances.  Candidates arrive in no particular order; every later step is order
+// Pruned search over per-point candidate lists (see gemm_candidates_kernel).  The first test of a batch
+// filters the point's candidates that belong to the batch with the exact threshold best * ratios[d'].
+// Candidates arrive in no particular order inside a batch; every later step is order
 // independent (thresholds are fixed inside a batch, the final minimum breaks ties by position).
 // Batches that hold no candidate are skipped: they would prune everything (count 0) anyway.
-// Points whose list overflowed (count > cap) are left untouched for the dense path.
+// Points whose list overflowed (count > cap) are left untouched and reported to the caller.
 // ---------------------------------------------------------------------------------------------
-struct PruneListArgs {
-    const uint2* cand;            // n_chunk x cap {centroid index, partial distance bits}
-    const uint32_t* cand_count;   // n_chunk
-    uint32_t cap;
-    const float* best0;           // seed distances
-    const float* x;
-    const float* pdx;
-    const float* aux;
-    const float* ratios;
-    uint32_t* idx;
-    float* dist;
-    uint32_t* not_pruned;
-    unsigned long long* stage_pairs;
-    const uint32_t* order;        // null, or the sequence in which the wavefronts take the points
-    uint64_t* over_ids;           // ids (id_offset + point) of the points whose list overflowed, appended here
-    uint32_t* n_over;             // their count
-    uint64_t id_offset;
-    int n, k, d, vertical_d, partial_d;
-};
 
 template <bool VEC, bool ACCT>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
 __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneListArgs a) {
@@ -678,6 +380,7 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     a.cand = cand; a.cand_count = cand_count; a.cap = cap; a.best0 = best0; a.x = x; a.pdx = pdx; a.aux = aux;
     a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
+    a.jb_lo = 0; a.jb_hi = 0x7fffffff; a.cursor = nullptr;  // one launch walks every batch
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
     dim3 grid(die_striped_groups(n_chunk, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (vec && d_stage_pairs)
@@ -701,26 +404,6 @@ int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, in
     if (m <= 0) return SKM_OK;
     hipLaunchKernelGGL(scatter_u32_kernel, dim3((m + 255) / 256), dim3(256), 0, ctx->stream, in, ids, m, out);
     return check_hip(hipGetLastError(), "scatter_u32_kernel launch");
-}
-
-int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
-                 const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
-                 int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
-                 uint32_t* out_not_pruned, unsigned long long* d_stage_pairs) {
-    if (n_chunk <= 0) return SKM_OK;
-    PruneArgs a;
-    a.partial = partial; a.ld_partial = ld_partial; a.x = x; a.c = c; a.pdx = pdx; a.aux = aux;
-    a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned;
-    a.stage_pairs = d_stage_pairs;
-    a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
-    const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) &&
-                     (reinterpret_cast<uintptr_t>(c) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
-    dim3 grid(die_striped_groups(n_chunk, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
-    if (vec)
-        hipLaunchKernelGGL(prune_kernel<true>, grid, block, 0, ctx->stream, a);
-    else
-        hipLaunchKernelGGL(prune_kernel<false>, grid, block, 0, ctx->stream, a);
-    return check_hip(hipGetLastError(), "prune_kernel launch");
 }
 
 } // namespace skm

@@ -1,6 +1,8 @@
 // Context, memory, error and profiler plumbing of libskm_hip.so.
 #include "skm_internal.h"
 
+#include <cstdlib>
+
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -32,15 +34,27 @@ int check_hip(hipError_t e, const char* what) {
 // Device blocks released by skm_free, by a context's workspace or by skm_ctx_destroy are kept and handed out
 // again: hipMalloc / hipFree of the gigabyte-sized buffers of a Train cost milliseconds each and hipFree waits
 // for the whole device.  One cache per device and process; a request takes the smallest cached block of at least
-// its size and at most 1/8 more.  The cache holds at most DEVICE_CACHE_MAX_BYTES and DEVICE_CACHE_MAX_BLOCKS
+// its size and at most 1/8 more.  The cache holds at most its byte limit and DEVICE_CACHE_MAX_BLOCKS
 // (beyond that a released block goes back to the driver), and is emptied when an allocation fails or on
 // skm_device_cache_trim.  A block enters the cache only after the releasing context's stream has drained.
 // ---------------------------------------------------------------------------------------------
 namespace {
-constexpr size_t DEVICE_CACHE_MAX_BYTES = size_t(96) << 30;
+constexpr size_t DEVICE_CACHE_DEFAULT_MAX_BYTES = size_t(48) << 30;
 constexpr size_t DEVICE_CACHE_MAX_BLOCKS = 2048;
+// Limit of the idle bytes: SKM_DEVICE_CACHE_BYTES in the environment when the process first uses a device, else the
+// default; skm_device_cache_set_limit changes it later.
+static size_t initial_cache_limit() {
+    const char* env = getenv("SKM_DEVICE_CACHE_BYTES");
+    if (env && *env) {
+        char* end = nullptr;
+        const unsigned long long v = strtoull(env, &end, 10);
+        if (end && *end == '\0') return (size_t) v;
+    }
+    return DEVICE_CACHE_DEFAULT_MAX_BYTES;
+}
 struct DeviceCache {
     std::mutex lock;
+    size_t max_bytes = initial_cache_limit();
     std::multimap<size_t, void*> idle;           // size -> block
     std::unordered_map<void*, size_t> size_of;   // every block handed out or idle
     size_t idle_bytes = 0;
@@ -91,7 +105,7 @@ int device_release(int device, void* ptr) {
     const auto known = c.size_of.find(ptr);
     if (known == c.size_of.end()) return check_hip(hipFree(ptr), "hipFree");  // not one of ours
     const size_t bytes = known->second;
-    if (c.idle.size() >= DEVICE_CACHE_MAX_BLOCKS || c.idle_bytes + bytes > DEVICE_CACHE_MAX_BYTES) {
+    if (c.idle.size() >= DEVICE_CACHE_MAX_BLOCKS || c.idle_bytes + bytes > c.max_bytes) {
         c.size_of.erase(known);
         return check_hip(hipFree(ptr), "hipFree");
     }
@@ -327,10 +341,36 @@ int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which) {
     return SKM_OK;
 }
 
+int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(which >= 0 && which <= 2, "which must be 0 (automatic), 1 (one point per wavefront) or 2 (pooled)");
+    ctx->walk_kernel = which;
+    return SKM_OK;
+}
+
+int skm_ctx_set_walk_launches(skm_ctx* ctx, int launches) {
+    SKM_REQUIRE(ctx, "null context");
+    SKM_REQUIRE(launches >= 1, "launches must be at least 1");
+    ctx->walk_launches = launches;
+    return SKM_OK;
+}
+
 int skm_malloc(skm_ctx* ctx, size_t bytes, void** out_d_ptr) {
     SKM_REQUIRE(ctx && out_d_ptr, "null argument");
     SKM_HIP_TRY(hipSetDevice(ctx->device));
     return device_alloc(ctx->device, bytes, out_d_ptr);
+}
+
+int skm_device_cache_set_limit(int device, size_t bytes) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || device < 0 || device >= n)
+        return set_error(SKM_ERR_INVALID, "skm_device_cache_set_limit: no such device");
+    SKM_HIP_TRY(hipSetDevice(device));
+    DeviceCache& c = device_cache(device);
+    std::lock_guard<std::mutex> guard(c.lock);
+    c.max_bytes = bytes;
+    if (c.idle_bytes > bytes) trim_locked(c);
+    return SKM_OK;
 }
 
 int skm_device_cache_trim(int device) {

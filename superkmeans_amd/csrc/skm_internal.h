@@ -29,6 +29,8 @@ struct skm_ctx {
     unsigned copy_seq = 0;
     size_t workspace_limit = size_t(24) << 30;
     int candidate_kernel = 0;  // skm_ctx_set_candidate_kernel
+    int walk_kernel = 0;       // skm_ctx_set_walk_kernel
+    int walk_launches = 1;     // skm_ctx_set_walk_launches
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
     static constexpr int WS_SLOTS = 6;
     void* ws[WS_SLOTS] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -132,10 +134,6 @@ int launch_merge_granules(skm_ctx* ctx, const uint2* granule_min, int n, int k, 
 
 // Number of striped copies of the per-stage accounting counters (each n_hblocks + 2 entries long).
 constexpr int SKM_ACCT_COPIES = 64;
-int launch_prune(skm_ctx* ctx, const float* partial, int64_t ld_partial, const float* x, int n_chunk,
-                 const float* c, const float* pdx, const float* aux, int k, int d, int vertical_d,
-                 int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist,
-                 uint32_t* out_not_pruned, unsigned long long* d_stage_pairs);
 
 int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                            const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
@@ -155,6 +153,15 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
                       uint64_t id_offset);
+// The same walk with several points per wavefront (rows 16-byte aligned, d a multiple of 4); `serves` says whether a
+// call qualifies.  Same results bit for bit.  One launch walks the batches [jb_lo, jb_hi) of 1024 centroids; a walk
+// split over several launches (ascending ranges) keeps its place in `cursor` (n_chunk words).
+bool prune_pool_serves(const float* x, const float* pdx, int d);
+int launch_prune_pool(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
+                      const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
+                      int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
+                      unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
+                      uint64_t id_offset, int jb_lo, int jb_hi, uint32_t* cursor);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 

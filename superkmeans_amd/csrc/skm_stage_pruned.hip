@@ -6,10 +6,10 @@
 //   2. gemm_candidates_kernel or gemm_candidates_stationary_kernel (d' up to 160 and enough points to fill the
 //                               chip with 256-point workgroups): MFMA partial distances; the epilogue emits only
 //                               pairs below thr0 into per-point lists (nothing dense is written)
-//   3. prune_list_kernel        exact per-batch thresholds, block-wise pruning, best candidate
+//   3. prune_pool_kernel (rows 16-byte aligned) or prune_list_kernel: exact per-batch thresholds, block-wise
+//                               pruning, best candidate
 // After the last chunk, the points whose list overflowed (loose seeds, points with no centroid nearby)
-// are gathered and redone with the dense pair gemm_store_kernel + prune_kernel: same results, more
-// traffic, and only for those points.
+// are gathered and go through the same three kernels once more with lists long enough for every centroid.
 #include "skm_internal.h"
 
 #include <algorithm>
@@ -28,50 +28,95 @@ namespace {
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// Dense path on a contiguous block of points (also the fallback for overflowed points).
-int dense_block(skm_ctx* ctx, const float* d_x, size_t m, const float* d_c, const float* d_pdx, const float* d_aux,
-                size_t k, size_t d, size_t vertical_d, uint32_t partial_d, const float* d_ratios, const float* d_xnorm_p,
-                const float* d_cnorm_p, uint32_t* d_idx, float* d_dist, uint32_t* d_counts, unsigned long long* d_stage) {
-    const size_t ld = align_up(k, 64);
-    size_t sub = ctx->workspace_limit / (ld * sizeof(float));
-    sub = std::max<size_t>(128, (sub / 128) * 128);
-    sub = std::min<size_t>(sub, size_t(1) << 22);
-    void* ws_partial = nullptr;
-    SKM_TRY(workspace(ctx, 0, std::min(sub, m) * ld * sizeof(float), &ws_partial));
-    for (size_t i0 = 0; i0 < m; i0 += sub) {
-        const size_t mm = std::min(sub, m - i0);
-        {
-            ScopedStage st(ctx, "search/overflow/blas");
-            SKM_TRY(launch_gemm_store(ctx, d_x + i0 * d, (int) mm, (int64_t) d, d_c, (int) k, (int64_t) d, (int) partial_d,
-                                      (float*) ws_partial, (int64_t) ld, d_xnorm_p + i0, d_cnorm_p));
-        }
-        {
-            ScopedStage st(ctx, "search/overflow/pdx");
-            SKM_TRY(launch_prune(ctx, (const float*) ws_partial, (int64_t) ld, d_x + i0 * d, (int) mm, d_c, d_pdx, d_aux,
-                                 (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_idx + i0, d_dist + i0,
-                                 d_counts + i0, d_stage));
-        }
+struct SearchOperands {
+    const float *d_c, *d_pdx, *d_aux, *d_ratios, *d_cnorm_p;
+    size_t k, d, vertical_d;
+    uint32_t partial_d;
+};
+
+// Seed, candidate lists and list walk of one chunk of m points whose lists have `cap` slots each.  Points whose list
+// overflows are left untouched and appended to d_over_ids (as id_offset + row).
+int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t m, const float* d_xnorm_p, uint32_t cap,
+                 uint2* d_cand, float* d_best0, float* d_thr0, uint32_t* d_cand_count, uint32_t* d_inout_idx, float* d_out_dist,
+                 uint32_t* d_counts, unsigned long long* stage_arg, const uint32_t* order, uint64_t* d_over_ids,
+                 uint32_t* d_n_over, uint64_t id_offset, bool zero_n_over, bool long_lists, uint32_t* d_cursor,
+                 const char* scope_seed, const char* scope_blas, const char* scope_pdx) {
+    {
+        ScopedStage st(ctx, scope_seed);
+        SKM_TRY(launch_seed_distance(ctx, xc, o.d_c, d_inout_idx, (int) m, (int) o.d, o.d_ratios, (int) o.partial_d, d_best0,
+                                     d_thr0, order, zero_n_over ? d_n_over : (uint32_t*) nullptr));
+    }
+    {
+        ScopedStage st(ctx, scope_blas);
+        // the register-stationary kernel addresses the 64 lists of a wavefront with 32-bit byte offsets
+        const bool lists_fit = (uint64_t) cap * 64 * sizeof(uint2) < (uint64_t(1) << 32);
+        if (ctx->candidate_kernel != 1 && lists_fit &&
+            gemm_candidates_stationary_serves(o.d_c, (int) o.k, xc, (int) m, (int) o.partial_d, (int64_t) o.d,
+                                              ctx->candidate_kernel == 2))
+            SKM_TRY(launch_gemm_candidates_stationary(ctx, o.d_c, (int) o.k, xc, (int) m, (int) o.partial_d, (int64_t) o.d,
+                                                      d_xnorm_p, o.d_cnorm_p, d_thr0, d_cand_count, d_cand, cap));
+        else
+            SKM_TRY(launch_gemm_candidates(ctx, o.d_c, (int) o.k, xc, (int) m, (int) o.partial_d, (int64_t) o.d, d_xnorm_p,
+                                           o.d_cnorm_p, d_thr0, d_cand_count, d_cand, cap));
+    }
+    {
+        ScopedStage st(ctx, scope_pdx);
+        // Several points per wavefront pay when the lists are short and the points many: with few points the chip is
+        // not filled by an eighth as many wavefronts, and a long list fills the passes of its point by itself.
+        const bool pooled = ctx->walk_kernel != 1 && prune_pool_serves(xc, o.d_pdx, (int) o.d) &&
+                            (ctx->walk_kernel == 2 || (!long_lists && m >= 32768));
+        if (pooled) {
+            const int n_batches = (int) ((o.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE);
+            const int phases = std::max(1, std::min(ctx->walk_launches, n_batches));
+            for (int ph = 0; ph < phases; ++ph) {
+                const int lo = (int) ((int64_t) n_batches * ph / phases), hi = (int) ((int64_t) n_batches * (ph + 1) / phases);
+                SKM_TRY(launch_prune_pool(ctx, d_cand, d_cand_count, cap, d_best0, xc, (int) m, o.d_pdx, o.d_aux, (int) o.k,
+                                          (int) o.d, (int) o.vertical_d, (int) o.partial_d, o.d_ratios, d_inout_idx, d_out_dist,
+                                          d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset, lo, hi, d_cursor));
+            }
+        } else
+            SKM_TRY(launch_prune_list(ctx, d_cand, d_cand_count, cap, d_best0, xc, (int) m, o.d_pdx, o.d_aux, (int) o.k,
+                                      (int) o.d, (int) o.vertical_d, (int) o.partial_d, o.d_ratios, d_inout_idx, d_out_dist,
+                                      d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset));
     }
     return SKM_OK;
 }
 
-// Dense search of the points `d_ids` from their seeds in d_inout_idx: gather, dense partial distances + dense pruning
-// over all batches, results scattered back.
-int dense_redo(skm_ctx* ctx, int slot, const float* d_x, const uint64_t* d_ids, size_t mo, const float* d_c, const float* d_pdx,
-               const float* d_aux, size_t k, size_t d, size_t vertical_d, uint32_t partial_d, const float* d_ratios,
-               const float* d_xnorm_p, const float* d_cnorm_p, uint32_t* d_inout_idx, float* d_out_dist, uint32_t* d_counts,
-               unsigned long long* d_stage) {
+// The points `d_ids`, whose lists overflowed, searched again from the same seeds with lists that hold every centroid:
+// rows, norms and seeds are gathered into a compact block, the block goes through the same three kernels in chunks
+// that fit the workspace, results are scattered back.  Same candidates, same thresholds, same walk: same results as
+// lists of that length would have given in the first place.
+int redo_with_full_lists(skm_ctx* ctx, const SearchOperands& o, const float* d_x, const uint64_t* d_ids, size_t mo,
+                         const float* d_xnorm_p, uint32_t* d_inout_idx, float* d_out_dist, uint32_t* d_counts,
+                         unsigned long long* stage_arg) {
+    const uint32_t cap = (uint32_t) align_up(o.k, 64);
+    size_t chunk = ctx->workspace_limit / (size_t(cap) * sizeof(uint2));
+    chunk = std::max<size_t>(128, (chunk / 128) * 128);
+    chunk = std::min(chunk, align_up(mo, 128));
+    const size_t mo_pad = align_up(mo, 64);
     void* ws_o = nullptr;
-    SKM_TRY(workspace(ctx, slot, mo * d * sizeof(float) + 4 * align_up(mo, 64) * sizeof(uint32_t) + 256, &ws_o));
-    float* xo = (float*) ws_o;
-    float* xnorm_o = xo + mo * d;
-    uint32_t* idx_o = (uint32_t*) (xnorm_o + align_up(mo, 64));
-    float* dist_o = (float*) (idx_o + align_up(mo, 64));
-    uint32_t* cnt_o = (uint32_t*) (dist_o + align_up(mo, 64));
-    SKM_TRY(skm_gather_rows(ctx, d_x, d, d_ids, mo, xo, d_xnorm_p, xnorm_o));
+    SKM_TRY(workspace(ctx, 3, mo * o.d * sizeof(float) + (8 * mo_pad + 64) * sizeof(uint32_t) + mo_pad * sizeof(uint64_t), &ws_o));
+    uint64_t* over2 = (uint64_t*) ws_o;  // never filled: no list overflows
+    float* xo = (float*) (over2 + mo_pad);
+    float* xnorm_o = xo + mo * o.d;
+    uint32_t* idx_o = (uint32_t*) (xnorm_o + mo_pad);
+    float* dist_o = (float*) (idx_o + mo_pad);
+    uint32_t* cnt_o = (uint32_t*) (dist_o + mo_pad);
+    float* best0_o = (float*) (cnt_o + mo_pad);
+    float* thr0_o = best0_o + mo_pad;
+    uint32_t* cand_count_o = (uint32_t*) (thr0_o + mo_pad);
+    uint32_t* cursor_o = cand_count_o + mo_pad;
+    uint32_t* n_over2 = cursor_o + mo_pad;  // stays 0
+    SKM_TRY(skm_gather_rows(ctx, d_x, o.d, d_ids, mo, xo, d_xnorm_p, xnorm_o));
     SKM_TRY(launch_gather_u32(ctx, d_inout_idx, d_ids, (int) mo, idx_o));
-    SKM_TRY(dense_block(ctx, xo, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, xnorm_o, d_cnorm_p, idx_o, dist_o,
-                        cnt_o, d_stage));
+    for (size_t i0 = 0; i0 < mo; i0 += chunk) {
+        const size_t m = std::min(chunk, mo - i0);
+        void* ws_cand = nullptr;
+        SKM_TRY(workspace(ctx, 0, m * size_t(cap) * sizeof(uint2), &ws_cand));
+        SKM_TRY(search_chunk(ctx, o, xo + i0 * o.d, m, xnorm_o + i0, cap, (uint2*) ws_cand, best0_o + i0, thr0_o + i0,
+                             cand_count_o + i0, idx_o + i0, dist_o + i0, cnt_o + i0, stage_arg, nullptr, over2, n_over2, i0,
+                             i0 == 0, true, cursor_o + i0, "search/overflow/seed", "search/overflow/blas", "search/overflow/pdx"));
+    }
     SKM_TRY(launch_scatter_u32(ctx, idx_o, d_ids, (int) mo, d_inout_idx));
     SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_ids, (int) mo, (uint32_t*) d_out_dist));
     SKM_TRY(launch_scatter_u32(ctx, cnt_o, d_ids, (int) mo, d_counts));
@@ -110,9 +155,10 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     const size_t cn = std::min(chunk, n);
 
     void* ws_counts = nullptr;
-    SKM_TRY(workspace(ctx, 1, n * sizeof(uint32_t) + SKM_ACCT_COPIES * (n_hblocks + 2) * sizeof(unsigned long long) + 64, &ws_counts));
+    SKM_TRY(workspace(ctx, 1, 2 * n * sizeof(uint32_t) + SKM_ACCT_COPIES * (n_hblocks + 2) * sizeof(unsigned long long) + 64, &ws_counts));
     unsigned long long* d_stage = (unsigned long long*) ws_counts;
     uint32_t* d_counts = (uint32_t*) (d_stage + SKM_ACCT_COPIES * (n_hblocks + 2));
+    uint32_t* d_cursor = d_counts + n;  // place of every point in its list, for a walk split over several launches
     if (h_out_stage_pairs) SKM_TRY(skm_fill_u32(ctx, d_stage, 0u, 2 * SKM_ACCT_COPIES * (n_hblocks + 2)));
     unsigned long long* stage_arg = h_out_stage_pairs ? d_stage : nullptr;
 
@@ -127,37 +173,17 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
 
     // The order the last centroid update left, when it covers exactly these points and they are one chunk.
     const uint32_t* order = (chunk >= n && ctx->cluster_order_n == n) ? ctx->cluster_order : nullptr;
+    const SearchOperands o{d_c, d_pdx, d_aux, d_ratios, d_cnorm_p, k, d, vertical_d, partial_d};
     for (size_t i0 = 0; i0 < n; i0 += chunk) {
         const size_t m = std::min(chunk, n - i0);
         void* ws_cand = nullptr;
         SKM_TRY(workspace(ctx, 0, m * size_t(cap) * sizeof(uint2), &ws_cand));
-        const float* xc = d_x + i0 * d;
-        {
-            ScopedStage st(ctx, "search/seed");
-            SKM_TRY(launch_seed_distance(ctx, xc, d_c, d_inout_idx + i0, (int) m, (int) d, d_ratios, (int) partial_d,
-                                         d_best0, d_thr0, order, i0 == 0 ? d_n_over : (uint32_t*) nullptr));
-        }
-        {
-            ScopedStage st(ctx, "search/blas");
-            if (ctx->candidate_kernel != 1 &&
-                gemm_candidates_stationary_serves(d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d,
-                                                  ctx->candidate_kernel == 2))
-                SKM_TRY(launch_gemm_candidates_stationary(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d,
-                                                          d_xnorm_p + i0, d_cnorm_p, d_thr0, d_cand_count,
-                                                          (uint2*) ws_cand, cap));
-            else
-                SKM_TRY(launch_gemm_candidates(ctx, d_c, (int) k, xc, (int) m, (int) partial_d, (int64_t) d, d_xnorm_p + i0,
-                                               d_cnorm_p, d_thr0, d_cand_count, (uint2*) ws_cand, cap));
-        }
-        {
-            ScopedStage st(ctx, "search/pdx");
-            SKM_TRY(launch_prune_list(ctx, (const uint2*) ws_cand, d_cand_count, cap, d_best0, xc, (int) m, d_pdx, d_aux,
-                                      (int) k, (int) d, (int) vertical_d, (int) partial_d, d_ratios, d_inout_idx + i0,
-                                      d_out_dist + i0, d_counts + i0, stage_arg, order, d_over_ids, d_n_over, (uint64_t) i0));
-        }
+        SKM_TRY(search_chunk(ctx, o, d_x + i0 * d, m, d_xnorm_p + i0, cap, (uint2*) ws_cand, d_best0, d_thr0, d_cand_count,
+                             d_inout_idx + i0, d_out_dist + i0, d_counts + i0, stage_arg, order, d_over_ids, d_n_over,
+                             (uint64_t) i0, i0 == 0, false, d_cursor + i0, "search/seed", "search/blas", "search/pdx"));
     }
-    // Points whose list overflowed (loose seeds, or points with no centroid nearby): one dense redo for
-    // all of them: gather, dense partial distances + dense pruning, scatter the results back.  The sum of the
+    // Points whose list overflowed (loose seeds, or points with no centroid nearby) are searched again with lists that
+    // hold every centroid.  The sum of the
     // per-point counts is queued before the number of overflowing points is known and both arrive with one wait;
     // it is taken again only if a redo changed some counts.
     double* h_not_pruned = nullptr;
@@ -173,8 +199,7 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     const size_t mo = *(volatile uint32_t*) h_n_over;
     if (mo > 0) {
         ScopedStage st(ctx, "search/overflow");
-        SKM_TRY(dense_redo(ctx, 3, d_x, d_over_ids, mo, d_c, d_pdx, d_aux, k, d, vertical_d, partial_d, d_ratios, d_xnorm_p,
-                           d_cnorm_p, d_inout_idx, d_out_dist, d_counts, stage_arg));
+        SKM_TRY(redo_with_full_lists(ctx, o, d_x, d_over_ids, mo, d_xnorm_p, d_inout_idx, d_out_dist, d_counts, stage_arg));
     }
     if (h_out_not_pruned) {
         double total = *(volatile double*) h_not_pruned;

@@ -11,8 +11,9 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, kernel=0):
-    """kernel: skm_ctx_set_candidate_kernel (0 automatic, 1 tiled, 2 register-stationary where the shape allows)."""
+def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, kernel=0, walk=0, launches=1):
+    """kernel: skm_ctx_set_candidate_kernel (0 automatic, 1 tiled, 2 register-stationary where the shape allows);
+    walk: skm_ctx_set_walk_kernel (0 automatic, 1 one point per wavefront, 2 pooled wherever rows are aligned)."""
     n, d = X.shape
     k = C.shape[0]
     H, V = oracle.dimension_split(d)
@@ -27,12 +28,16 @@ def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, 
     total = ctypes.c_uint64()
     stages = (ctypes.c_uint64 * (H // 64 + 2))()
     capi.check(ctx.lib.skm_ctx_set_candidate_kernel(ctx.handle, kernel))
+    capi.check(ctx.lib.skm_ctx_set_walk_kernel(ctx.handle, walk))
+    capi.check(ctx.lib.skm_ctx_set_walk_launches(ctx.handle, launches))
     try:
         capi.check(ctx.lib.skm_assign_pruned(ctx.handle, dX.ptr, n, dC.ptr, dP.ptr, dA.ptr, k, d, V, partial_d, dR.ptr,
                                              xn.ptr, cn.ptr, idx.ptr, dist.ptr, ctypes.byref(total),
                                              stages if accounting else None))
     finally:
         capi.check(ctx.lib.skm_ctx_set_candidate_kernel(ctx.handle, 0))
+        capi.check(ctx.lib.skm_ctx_set_walk_kernel(ctx.handle, 0))
+        capi.check(ctx.lib.skm_ctx_set_walk_launches(ctx.handle, 1))
     out = idx.download(), dist.download(), total.value, np.array(list(stages), dtype=np.uint64)
     for a in (dX, dC, dP, dA, xn, cn, dR, idx, dist):
         a.free()
@@ -115,9 +120,63 @@ def test_both_candidate_kernels_give_the_same_bits(capi, ctx, oracle, blobs, n, 
     assert np.sum(gi != oi) <= max(1, int(1e-4 * n))
 
 
+def _same_bits(a, b):
+    assert np.array_equal(a[0], b[0])
+    assert np.array_equal(a[1].view(np.uint32), b[1].view(np.uint32))
+    assert a[2] == b[2]
+    assert np.array_equal(a[3], b[3])
+
+
+# The two list walks (one point per wavefront; eight points pooled per wavefront): same assignments, same distance
+# bits, same not-pruned totals and, with accounting, the same pairs entering every step.  Shapes: one batch and many,
+# a last batch of a few centroids, point counts that leave the last wavefront with one to seven points, tight seeds
+# (few survivors: the few-entry path) and random seeds (hundreds of survivors per batch: pool rounds, overflowing lists).
+@pytest.mark.parametrize("n,d,k,partial_d,random_seeds", [(4000, 128, 300, 32, False), (6001, 256, 1500, 32, False),
+                                                          (3003, 768, 1100, 96, False), (4000, 1024, 2500, 128, False),
+                                                          (1502, 600, 1030, 76, False), (1000, 132, 260, 23, False),
+                                                          (2050, 256, 1500, 32, True), (1237, 768, 3100, 64, True),
+                                                          (9, 128, 20, 16, False), (3, 256, 1100, 16, True),
+                                                          (2500, 512, 5000, 48, True)])
+@pytest.mark.parametrize("accounting", [False, True])
+def test_both_list_walks_give_the_same_bits(capi, ctx, oracle, blobs, n, d, k, partial_d, random_seeds, accounting):
+    X, C, prev = _setup(oracle, blobs, max(n, k + 10), d, k, seed=3 * n + d + partial_d)
+    X, prev = X[:n], prev[:n]
+    if random_seeds:
+        prev = np.random.default_rng(n).integers(0, k, n).astype(np.uint32)
+    ratios = oracle.ratios(d, 1.5)
+    single = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=1)
+    pooled = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=2)
+    _same_bits(single, pooled)
+    # the pooled walk split into one launch per batch, or per range of batches, resumes from the state the launch before left
+    for launches in (2, 1000):
+        split = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=2, launches=launches)
+        _same_bits(single, split)
+
+
+def test_both_list_walks_with_loose_ratios(capi, ctx, oracle, blobs):
+    """Loose ratios: nearly every candidate survives many blocks, pools fill up (rounds over whole points, a point
+    alone filling most of a pool) and most lists overflow into the pass with full-length lists."""
+    n, d, k = 3000, 256, 2600
+    X, C, _ = _setup(oracle, blobs, n, d, k, seed=11)
+    prev = np.random.default_rng(3).integers(0, k, n).astype(np.uint32)
+    ratios = np.minimum(1.0, 3.0 * oracle.ratios(d, 1.5)).astype(np.float32)
+    ratios[d] = 1.0
+    for accounting in (False, True):
+        single = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, accounting=accounting, walk=1)
+        pooled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, accounting=accounting, walk=2)
+        _same_bits(single, pooled)
+    ones = np.ones(d + 1, dtype=np.float32)  # nothing is ever pruned: every pool is as full as it can get
+    single = _pruned(capi, ctx, oracle, X[:600], C, prev[:600], 40, ones, accounting=True, walk=1)
+    pooled = _pruned(capi, ctx, oracle, X[:600], C, prev[:600], 40, ones, accounting=True, walk=2)
+    _same_bits(single, pooled)
+    bi, bbest, bsecond = oracle.brute_force(X[:600], C)
+    tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+    assert np.all((pooled[0] == bi) | tie)
+
+
 def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs):
     """Random seeds at k > 1024: thresholds are loose, many points collect more candidates than their list holds
-    (cap = 1024 slots) and are redone densely; the two kernels must still agree bit for bit."""
+    (cap = 1024 slots) and are searched again with full-length lists; the two kernels must still agree bit for bit."""
     n, d, k = 3000, 256, 2600
     X, C, _ = _setup(oracle, blobs, n, d, k, seed=11)
     prev = np.random.default_rng(3).integers(0, k, n).astype(np.uint32)
