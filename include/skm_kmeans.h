@@ -94,6 +94,19 @@ int skm_kmeans_assign_device(skm_kmeans* km, const float* d_vectors, const float
 int skm_kmeans_assign_training_points(skm_kmeans* km, const float* h_vectors, const float* h_centroids,
                                       size_t n_vectors, size_t n_centroids, uint32_t* h_out_assignments);
 
+/* The centroid each of the vectors of the last skm_kmeans_assign_training_points started its pruned search from: the
+ * training assignment, a size-weighted draw or the representative of the nearest meso-centroid, by the branch of
+ * superkmeans.h:454-563 (the reference builds them in place in its result array; kept here so that a binding's tests
+ * can compare them).  count must equal that call's n_vectors; SKM_ERR_RUNTIME when there was no such call or it fell
+ * back to Assign. */
+int skm_kmeans_get_training_seeds(skm_kmeans* km, uint32_t* h_out, size_t count);
+
+/* Test hook, no counterpart in the reference: SplitClusters of the object's class (flat: superkmeans.h:890-928;
+ * hierarchical: hierarchical_superkmeans.h:579-678) on a given state.  h_centroids (k x d) and h_sizes (k) are replaced
+ * by the edited rows and sizes, out_n_split receives the number of splits.  Untrained objects only. */
+int skm_kmeans_split_clusters_on_state(skm_kmeans* km, float* h_centroids, uint32_t* h_sizes, size_t k, size_t n_samples,
+                                       uint64_t* out_n_split);
+
 int skm_kmeans_get_n_clusters(skm_kmeans* km, size_t* out);
 int skm_kmeans_is_trained(skm_kmeans* km, int* out);
 /* which: 0 iteration_stats (flat), 1 mesoclustering, 2 fineclustering, 3 refinement. */

@@ -224,6 +224,7 @@ class SuperKMeans {
         if (!trained) {
             throw std::runtime_error("AssignTrainingPoints requires SuperKMeans to be trained first");
         }
+        training_seeds.clear();
         if (config.use_blas_only || d < DIMENSION_THRESHOLD_FOR_PRUNING ||
             n_clusters <= N_CLUSTERS_THRESHOLD_FOR_PRUNING) {
             if (!config.suppress_warnings) {
@@ -310,6 +311,7 @@ class SuperKMeans {
         }
         dbuf<uint32_t> d_seed(ctx, n_vectors);
         d_seed.Upload(seeds.data(), n_vectors);
+        training_seeds = std::move(seeds);
         dbuf<float> d_norms_p(ctx, n_vectors), d_dist(ctx, n_vectors);
         hip::Check(skm_norms(ctx, d_rot.get(), n_vectors, d, partial_d, d_norms_p.get()));
         uint64_t not_pruned_total = 0;
@@ -331,6 +333,30 @@ class SuperKMeans {
 
     [[nodiscard]] size_t GetNClusters() const noexcept { return n_clusters; }
     [[nodiscard]] bool IsTrained() const noexcept { return trained; }
+    /**
+     * Test hook, no counterpart in the reference: SplitClusters of this object's class (the flat rule here,
+     * superkmeans.h:890-928; the balancing rule in HierarchicalSuperKMeans, hierarchical_superkmeans.h:579-678) applied
+     * to a given state, so that its decisions and row arithmetic can be compared with another implementation's on
+     * hand-made states.  h_centroids (k x d) and h_sizes (k) are replaced by the edited rows and sizes; returns the
+     * number of splits.  Untrained objects only (it overwrites the object's centroid buffers).
+     */
+    size_t SplitClustersOnState(centroid_value_t* h_centroids, uint32_t* h_sizes, const size_t k, const size_t n_samples_) {
+        if (trained) throw std::runtime_error("SplitClustersOnState needs an untrained object");
+        SKMEANS_ENSURE_POSITIVE(k);
+        horizontal_centroids.Reset(ctx, k * d);
+        horizontal_centroids.Upload(h_centroids, k * d);
+        cluster_sizes.reset(new uint32_t[k]);
+        std::memcpy(cluster_sizes.get(), h_sizes, k * sizeof(uint32_t));
+        SplitClusters(n_samples_, k);
+        horizontal_centroids.Download(h_centroids, k * d);
+        std::memcpy(h_sizes, cluster_sizes.get(), k * sizeof(uint32_t));
+        return n_split;
+    }
+
+    /** The centroid every vector of the last AssignTrainingPoints started its pruned search from (the reference
+     *  builds them in place in its result array, superkmeans.h:454-563); empty before the first call and after a
+     *  call that fell back to Assign. */
+    [[nodiscard]] const std::vector<uint32_t>& GetTrainingSeeds() const noexcept { return training_seeds; }
     [[nodiscard]] float GetSamplingFraction() const noexcept { return config.sampling_fraction; }
     /** Host copy of the per-point squared distances of the last training iteration. */
     [[nodiscard]] distance_t* GetDistancesPointer() { return host_distances.data(); }
@@ -1049,6 +1075,7 @@ class SuperKMeans {
     dbuf<float> rotated_queries, query_norms, gt_distances, recall_distances;
     dbuf<uint32_t> gt_assignments, promising_centroids;
     std::vector<float> host_distances;
+    std::vector<uint32_t> training_seeds;  // GetTrainingSeeds
     std::vector<centroid_value_t> prepared_centroids;  // PrepareHostOutputs
     std::thread host_outputs_thread;
     bool collect_prune_accounting = false;

@@ -84,6 +84,7 @@ def load():
     lib.oracle_horizontal.restype = c_float
     lib.oracle_kmeans_n_stats.restype = c_size_t
     lib.oracle_kmeans_n_samples.restype = c_size_t
+    lib.oracle_kmeans_last_seeds.restype = c_size_t
     lib.oracle_kmeans_accounting.restype = c_size_t
     lib.oracle_split_clusters.restype = c_size_t
     lib.oracle_n_mesoclusters.restype = c_size_t
@@ -392,6 +393,13 @@ class KMeans:
         sizes = np.empty(self.k, dtype=np.uint32)
         self.lib.oracle_kmeans_state(self.h, _fp(c), _fp(a), _fp(dist), _fp(sizes))
         return c, a, dist, sizes
+
+    def training_seeds(self):
+        """Seeds of the last assign_training_points (test hook of the restatement)."""
+        n = self.lib.oracle_kmeans_last_seeds(self.h, None, c_size_t(0))
+        out = np.empty(n, dtype=np.uint32)
+        self.lib.oracle_kmeans_last_seeds(self.h, _fp(out), c_size_t(n))
+        return out
 
     def collect_accounting(self, on=True):
         self.lib.oracle_kmeans_collect_accounting(self.h, c_int(1 if on else 0))

@@ -852,6 +852,7 @@ class KMeans {
         PDXIndex pdx_centroids;
         pdx_centroids.FromBuffer(centroids.get(), n_clusters, d, partial_horizontal_centroids.get(), pruner->ratios.data());
         if (config.sampling_fraction == 1.0f) {
+            last_seeds.assign(assignments.get(), assignments.get() + n_vectors);
             GetPartialL2NormsRowMajor(data_p, n_vectors, data_norms.get(), partial_d);
             FindNearestNeighborWithPruning(data_p, horizontal_centroids.get(), n_vectors, n_clusters, d,
                                            data_norms.get(), centroid_norms.get(), assignments.get(), distances.get(),
@@ -867,6 +868,7 @@ class KMeans {
             std::discrete_distribution<uint32_t> cluster_dist(cluster_sizes.get(), cluster_sizes.get() + n_clusters);
             for (; cur_vector_idx < n_vectors; ++cur_vector_idx)
                 result_assignments[sampled_indices[cur_vector_idx]] = cluster_dist(rng);
+            last_seeds = result_assignments;
             data_norms.reset(new float[n_vectors]);
             GetPartialL2NormsRowMajor(data_p, n_vectors, data_norms.get(), partial_d);
             FindNearestNeighborWithPruning(data_p, horizontal_centroids.get(), n_vectors, n_clusters, d,
@@ -899,6 +901,7 @@ class KMeans {
                 size_t orig_idx = sampled_indices[cur_vector_idx];
                 result_assignments[orig_idx] = meso_to_original[meso_assignments[orig_idx]];
             }
+            last_seeds = result_assignments;
             data_norms.reset(new float[n_vectors]);
             GetPartialL2NormsRowMajor(data_p, n_vectors, data_norms.get(), partial_d);
             FindNearestNeighborWithPruning(data_p, horizontal_centroids.get(), n_vectors, n_clusters, d,
@@ -937,6 +940,10 @@ class KMeans {
         c.dct_rotation = 0;
         return c;
     }
+
+    // Test hook, no counterpart in the reference: the seeds of the last AssignTrainingPoints, which the reference
+    // builds in place in its result array before the pruned search overwrites them.
+    std::vector<uint32_t> last_seeds;
 
     // ---- members mirrored from superkmeans.h:1445-1492 ----
     const size_t d;
@@ -1757,6 +1764,11 @@ void oracle_kmeans_state(void* h, float* out_rotated_centroids, uint32_t* out_as
     if (out_assignments) std::memcpy(out_assignments, km->assignments.get(), sizeof(uint32_t) * km->n_samples);
     if (out_distances) std::memcpy(out_distances, km->distances.get(), sizeof(float) * km->n_samples);
     if (out_cluster_sizes) std::memcpy(out_cluster_sizes, km->cluster_sizes.get(), sizeof(uint32_t) * km->n_clusters);
+}
+size_t oracle_kmeans_last_seeds(void* h, uint32_t* out, size_t cap) {
+    const auto& s = static_cast<KMeans*>(h)->last_seeds;
+    if (out && cap >= s.size()) std::memcpy(out, s.data(), s.size() * sizeof(uint32_t));
+    return s.size();
 }
 size_t oracle_kmeans_n_samples(void* h) { return static_cast<KMeans*>(h)->n_samples; }
 void oracle_kmeans_collect_accounting(void* h, int on) { static_cast<KMeans*>(h)->collect_accounting = on != 0; }

@@ -29,6 +29,7 @@ _PROTOTYPES = {
     "skm_ctx_set_candidate_kernel": (c_int, [c_void_p, c_int]),
     "skm_ctx_set_walk_kernel": (c_int, [c_void_p, c_int]),
     "skm_ctx_set_walk_launches": (c_int, [c_void_p, c_int]),
+    "skm_ctx_get_last_overflow": (c_int, [c_void_p, POINTER(c_uint64)]),
     "skm_malloc": (c_int, [c_void_p, c_size_t, POINTER(c_void_p)]),
     "skm_free": (c_int, [c_void_p, c_void_p]),
     "skm_device_cache_trim": (c_int, [c_int]),
@@ -90,6 +91,8 @@ _PROTOTYPES = {
     "skm_kmeans_n_stats": (c_int, [c_void_p, c_int, POINTER(c_size_t)]),
     "skm_kmeans_get_stats": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),
     "skm_kmeans_get_assignments": (c_int, [c_void_p, c_void_p, c_size_t]),
+    "skm_kmeans_get_training_seeds": (c_int, [c_void_p, c_void_p, c_size_t]),
+    "skm_kmeans_split_clusters_on_state": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, POINTER(c_uint64)]),
     "skm_kmeans_context": (c_int, [c_void_p, POINTER(c_void_p)]),
     "skm_kmeans_set_prune_accounting": (c_int, [c_void_p, c_int]),
     "skm_kmeans_get_prune_accounting": (
@@ -391,6 +394,20 @@ class KMeans:
     def assignments(self, count):
         out = np.empty(count, dtype=np.uint32)
         check(self.lib.skm_kmeans_get_assignments(self.handle, out.ctypes.data, count))
+        return out
+
+    def split_clusters_on_state(self, centroids, sizes, n_samples):
+        """SplitClusters of the object's class on a given state: returns (edited centroids, edited sizes, splits)."""
+        c = np.ascontiguousarray(centroids, dtype=np.float32).copy()
+        s = np.ascontiguousarray(sizes, dtype=np.uint32).copy()
+        n_split = c_uint64()
+        check(self.lib.skm_kmeans_split_clusters_on_state(self.handle, c.ctypes.data, s.ctypes.data, c.shape[0], n_samples,
+                                                          ctypes.byref(n_split)))
+        return c, s, int(n_split.value)
+
+    def training_seeds(self, count):
+        out = np.empty(count, dtype=np.uint32)
+        check(self.lib.skm_kmeans_get_training_seeds(self.handle, out.ctypes.data, count))
         return out
 
     @property

@@ -108,7 +108,11 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64) void seed_distance_kernel(
 // Points whose list overflowed (count > cap) are left untouched and reported to the caller.
 // ---------------------------------------------------------------------------------------------
 
-template <bool VEC, bool ACCT>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
+// DENSE: instead of a candidate list the point has a row of partial distances to all k centroids (a.partial), and the
+// first test of a batch scans the batch's 1024 entries of that row (InitPositionsArray, scalar_computers.h:87-98).
+// This serves the points whose list overflowed: for a point that a quarter of the centroids pass, writing and reading
+// the dense row is cheaper than appending and walking that many list entries.
+template <bool VEC, bool ACCT, bool DENSE>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
 __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneListArgs a) {
     // LIST_PAD slots past the live survivors: a pass of 32 gathers reads positions and adds partial sums without
     // asking whether a slot is live; the pad positions are kept at 0 (a valid centroid of any batch), what is added to
@@ -121,8 +125,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     const int p = point_of_wave(a.order, a.n, PRUNE_WAVES);
     if (p < 0) return;
     float* parts = s_parts[wave];
-    const uint32_t n_cand = a.cand_count[p];
-    if (n_cand > a.cap) {  // handled densely by the caller, who finds the point in the list of overflowing ones
+    const uint32_t n_cand = DENSE ? 0u : a.cand_count[p];
+    if (!DENSE && n_cand > a.cap) {  // handled by the caller, who finds the point in the list of overflowing ones
         if (lane == 0) a.over_ids[atomicAdd(a.n_over, 1u)] = a.id_offset + (uint64_t) p;
         return;
     }
@@ -135,6 +139,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     unsigned long long* acct = ACCT ? a.stage_pairs + (size_t) (blockIdx.x % SKM_ACCT_COPIES) * (n_hblocks + 2) : nullptr;
     const float* xq = a.x + (int64_t) p * d;
     const uint2* list = a.cand + (int64_t) p * a.cap;
+    const float* prow = DENSE ? a.partial + (int64_t) p * a.ld_partial : nullptr;
+    const int n_batches = (a.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE;
     const int sub = lane & 15, grp = lane >> 4;
 
     uint32_t best_idx = a.idx[p];
@@ -146,17 +152,31 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 5) void prune_list_kernel(PruneLi
     // the first entry not yet consumed.
     uint32_t chunk0 = 0, cur = 0;
     uint2 entry = make_uint2(0xffffffffu, 0u);
-    if (lane < n_cand) entry = list[lane];
+    if (!DENSE && lane < n_cand) entry = list[lane];
 
-    while (cur < n_cand) {
+    for (uint32_t jb_dense = 0; DENSE ? jb_dense < (uint32_t) n_batches : cur < n_cand; ++jb_dense) {
         // the same value in every lane: saying so keeps the batch's base pointers in scalar registers
-        const uint32_t jb = (uint32_t) __builtin_amdgcn_readfirstlane(__shfl((int) entry.x, (int) (cur - chunk0))) / SKM_Y_BATCH_SIZE;
+        const uint32_t jb = DENSE ? jb_dense
+                                  : (uint32_t) __builtin_amdgcn_readfirstlane(__shfl((int) entry.x, (int) (cur - chunk0))) / SKM_Y_BATCH_SIZE;
         const int base = (int) jb * SKM_Y_BATCH_SIZE;
         const int m = (a.k - base) < SKM_Y_BATCH_SIZE ? (a.k - base) : SKM_Y_BATCH_SIZE;
         const uint32_t prev_top_1 = best_idx;
         float thr = best * a.ratios[dp];
         int cnt = 0;
-        for (;;) {
+        for (int c0 = 0; DENSE && c0 < m; c0 += 64) {
+            const int c = c0 + lane;
+            const bool in = c < m;
+            const float v = in ? prow[base + c] : 0.0f;
+            const bool keep = in && (v < thr);
+            const unsigned long long mask = __ballot(keep);
+            if (keep) {
+                const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
+                pos[slot] = (uint16_t) c;
+                acc[slot] = v;
+            }
+            cnt += __popcll(mask);
+        }
+        for (; !DENSE;) {
             const uint32_t s = chunk0 + lane;
             const bool mine = s >= cur && s < n_cand && entry.x / SKM_Y_BATCH_SIZE == jb;
             const bool keep = mine && __uint_as_float(entry.y) < thr;
@@ -372,7 +392,7 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
-                      uint64_t id_offset) {
+                      uint64_t id_offset, const float* dense_partial, int64_t ld_partial) {
     if (n_chunk <= 0) return SKM_OK;
     PruneListArgs a;
     a.order = order;
@@ -381,16 +401,23 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     a.jb_lo = 0; a.jb_hi = 0x7fffffff; a.cursor = nullptr;  // one launch walks every batch
+    a.partial = dense_partial; a.ld_partial = ld_partial;
     const bool vec = (d % 4 == 0) && (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (reinterpret_cast<uintptr_t>(pdx) % 16 == 0);
     dim3 grid(die_striped_groups(n_chunk, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
-    if (vec && d_stage_pairs)
-        hipLaunchKernelGGL((prune_list_kernel<true, true>), grid, block, 0, ctx->stream, a);
-    else if (vec)
-        hipLaunchKernelGGL((prune_list_kernel<true, false>), grid, block, 0, ctx->stream, a);
-    else if (d_stage_pairs)
-        hipLaunchKernelGGL((prune_list_kernel<false, true>), grid, block, 0, ctx->stream, a);
-    else
-        hipLaunchKernelGGL((prune_list_kernel<false, false>), grid, block, 0, ctx->stream, a);
+#define SKM_LAUNCH_WALK(V, A, D) hipLaunchKernelGGL((prune_list_kernel<V, A, D>), grid, block, 0, ctx->stream, a)
+    const bool acct = d_stage_pairs != nullptr;
+    if (dense_partial) {
+        if (vec && acct) SKM_LAUNCH_WALK(true, true, true);
+        else if (vec) SKM_LAUNCH_WALK(true, false, true);
+        else if (acct) SKM_LAUNCH_WALK(false, true, true);
+        else SKM_LAUNCH_WALK(false, false, true);
+    } else {
+        if (vec && acct) SKM_LAUNCH_WALK(true, true, false);
+        else if (vec) SKM_LAUNCH_WALK(true, false, false);
+        else if (acct) SKM_LAUNCH_WALK(false, true, false);
+        else SKM_LAUNCH_WALK(false, false, false);
+    }
+#undef SKM_LAUNCH_WALK
     return check_hip(hipGetLastError(), "prune_list_kernel launch");
 }
 

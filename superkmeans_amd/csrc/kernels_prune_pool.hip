@@ -452,6 +452,7 @@ int launch_prune_pool(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     a.ratios = ratios; a.idx = inout_idx; a.dist = out_dist; a.not_pruned = out_not_pruned; a.stage_pairs = d_stage_pairs;
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     a.jb_lo = jb_lo; a.jb_hi = jb_hi; a.cursor = cursor;
+    a.partial = nullptr; a.ld_partial = 0;
     const int wavefronts = (n_chunk + POOL_PTS - 1) / POOL_PTS;
     dim3 grid(die_striped_groups(wavefronts, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
     if (d_stage_pairs)

@@ -108,6 +108,9 @@ struct PruneListArgs {
     // not_pruned and cursor as the launch over the batches before left them.  cursor: per point, entries consumed.
     int jb_lo, jb_hi;
     uint32_t* cursor;
+    // prune_list_kernel<.., DENSE> only: n x ld_partial partial distances to all centroids instead of the lists
+    const float* partial;
+    int64_t ld_partial;
 };
 
 } // namespace skm

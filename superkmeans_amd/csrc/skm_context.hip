@@ -348,6 +348,12 @@ int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which) {
     return SKM_OK;
 }
 
+int skm_ctx_get_last_overflow(skm_ctx* ctx, uint64_t* out_points) {
+    SKM_REQUIRE(ctx && out_points, "null argument");
+    *out_points = ctx->last_overflow_points;
+    return SKM_OK;
+}
+
 int skm_ctx_set_walk_launches(skm_ctx* ctx, int launches) {
     SKM_REQUIRE(ctx, "null context");
     SKM_REQUIRE(launches >= 1, "launches must be at least 1");

@@ -31,6 +31,7 @@ struct skm_ctx {
     int candidate_kernel = 0;  // skm_ctx_set_candidate_kernel
     int walk_kernel = 0;       // skm_ctx_set_walk_kernel
     int walk_launches = 1;     // skm_ctx_set_walk_launches
+    uint64_t last_overflow_points = 0;  // skm_ctx_get_last_overflow
     // Grow-only scratch buffers, one per role, so that stages never free inside a hot loop.
     static constexpr int WS_SLOTS = 6;
     void* ws[WS_SLOTS] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -145,6 +146,8 @@ int launch_gemm_candidates_stationary(skm_ctx* ctx, const float* C, int k, const
                                       const float* xnorm_p, const float* cnorm_p, const float* thr0,
                                       uint32_t* cand_count, uint2* cand, uint32_t cap);
 // `order`: null, or a permutation of the n points giving the sequence in which wavefronts take them.
+// launch_prune_list with dense_partial non-null: the points have rows of partial distances to all centroids
+// (n_chunk x ld_partial) instead of lists (cand, cand_count, over_ids and n_over are then unused).
 int launch_seed_distance(skm_ctx* ctx, const float* x, const float* c, const uint32_t* idx, int n, int d,
                          const float* ratios, int partial_d, float* best0, float* thr0, const uint32_t* order,
                          uint32_t* zero_this);
@@ -152,7 +155,7 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
-                      uint64_t id_offset);
+                      uint64_t id_offset, const float* dense_partial, int64_t ld_partial);
 // The same walk with several points per wavefront (rows 16-byte aligned, d a multiple of 4); `serves` says whether a
 // call qualifies.  Same results bit for bit.  One launch walks the batches [jb_lo, jb_hi) of 1024 centroids; a walk
 // split over several launches (ascending ranges) keeps its place in `cursor` (n_chunk words).

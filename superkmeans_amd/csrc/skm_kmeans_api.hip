@@ -187,6 +187,14 @@ int skm_kmeans_assign_training_points(skm_kmeans* km, const float* h_vectors, co
     });
 }
 
+int skm_kmeans_split_clusters_on_state(skm_kmeans* km, float* h_centroids, uint32_t* h_sizes, size_t k, size_t n_samples,
+                                       uint64_t* out_n_split) {
+    if (!km || !h_centroids || !h_sizes || !out_n_split)
+        return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_split_clusters_on_state: null argument");
+    if (n_samples <= k) return skm::set_error(SKM_ERR_INVALID, "skm_kmeans_split_clusters_on_state: n_samples must exceed k");
+    SKM_API_GUARD({ *out_n_split = km->base()->SplitClustersOnState(h_centroids, h_sizes, k, n_samples); });
+}
+
 int skm_kmeans_get_n_clusters(skm_kmeans* km, size_t* out) {
     if (!km || !out) return skm::set_error(SKM_ERR_INVALID, "null argument");
     *out = km->base()->GetNClusters();
@@ -239,6 +247,15 @@ int skm_kmeans_get_assignments(skm_kmeans* km, uint32_t* h_out, size_t count) {
     if (!km->base()->IsTrained()) return skm::set_error(SKM_ERR_RUNTIME, "the model has not been trained");
     if (count > km->n_trained) return skm::set_error(SKM_ERR_INVALID, "count exceeds the number of training points");
     std::memcpy(h_out, km->base()->assignments.get(), count * sizeof(uint32_t));
+    return SKM_OK;
+}
+
+int skm_kmeans_get_training_seeds(skm_kmeans* km, uint32_t* h_out, size_t count) {
+    if (!km || !h_out) return skm::set_error(SKM_ERR_INVALID, "null argument");
+    const std::vector<uint32_t>& seeds = km->base()->GetTrainingSeeds();
+    if (seeds.empty()) return skm::set_error(SKM_ERR_RUNTIME, "no pruned AssignTrainingPoints has run on this object");
+    if (count != seeds.size()) return skm::set_error(SKM_ERR_INVALID, "count differs from the number of vectors of that call");
+    std::memcpy(h_out, seeds.data(), count * sizeof(uint32_t));
     return SKM_OK;
 }
 

@@ -9,7 +9,8 @@
 //   3. prune_pool_kernel (rows 16-byte aligned) or prune_list_kernel: exact per-batch thresholds, block-wise
 //                               pruning, best candidate
 // After the last chunk, the points whose list overflowed (loose seeds, points with no centroid nearby)
-// are gathered and go through the same three kernels once more with lists long enough for every centroid.
+// are gathered and searched again through dense rows of partial distances (gemm_store_kernel with the distance
+// epilogue + the walk whose first test scans the row): same results, more traffic, and only for those points.
 #include "skm_internal.h"
 
 #include <algorithm>
@@ -39,15 +40,14 @@ struct SearchOperands {
 int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t m, const float* d_xnorm_p, uint32_t cap,
                  uint2* d_cand, float* d_best0, float* d_thr0, uint32_t* d_cand_count, uint32_t* d_inout_idx, float* d_out_dist,
                  uint32_t* d_counts, unsigned long long* stage_arg, const uint32_t* order, uint64_t* d_over_ids,
-                 uint32_t* d_n_over, uint64_t id_offset, bool zero_n_over, bool long_lists, uint32_t* d_cursor,
-                 const char* scope_seed, const char* scope_blas, const char* scope_pdx) {
+                 uint32_t* d_n_over, uint64_t id_offset, bool zero_n_over, uint32_t* d_cursor) {
     {
-        ScopedStage st(ctx, scope_seed);
+        ScopedStage st(ctx, "search/seed");
         SKM_TRY(launch_seed_distance(ctx, xc, o.d_c, d_inout_idx, (int) m, (int) o.d, o.d_ratios, (int) o.partial_d, d_best0,
                                      d_thr0, order, zero_n_over ? d_n_over : (uint32_t*) nullptr));
     }
     {
-        ScopedStage st(ctx, scope_blas);
+        ScopedStage st(ctx, "search/blas");
         // the register-stationary kernel addresses the 64 lists of a wavefront with 32-bit byte offsets
         const bool lists_fit = (uint64_t) cap * 64 * sizeof(uint2) < (uint64_t(1) << 32);
         if (ctx->candidate_kernel != 1 && lists_fit &&
@@ -60,11 +60,11 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
                                            o.d_cnorm_p, d_thr0, d_cand_count, d_cand, cap));
     }
     {
-        ScopedStage st(ctx, scope_pdx);
-        // Several points per wavefront pay when the lists are short and the points many: with few points the chip is
-        // not filled by an eighth as many wavefronts, and a long list fills the passes of its point by itself.
+        ScopedStage st(ctx, "search/pdx");
+        // Several points per wavefront pay when the points are many: with few points an eighth as many wavefronts
+        // do not fill the chip.
         const bool pooled = ctx->walk_kernel != 1 && prune_pool_serves(xc, o.d_pdx, (int) o.d) &&
-                            (ctx->walk_kernel == 2 || (!long_lists && m >= 32768));
+                            (ctx->walk_kernel == 2 || m >= 32768);
         if (pooled) {
             const int n_batches = (int) ((o.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE);
             const int phases = std::max(1, std::min(ctx->walk_launches, n_batches));
@@ -77,45 +77,61 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
         } else
             SKM_TRY(launch_prune_list(ctx, d_cand, d_cand_count, cap, d_best0, xc, (int) m, o.d_pdx, o.d_aux, (int) o.k,
                                       (int) o.d, (int) o.vertical_d, (int) o.partial_d, o.d_ratios, d_inout_idx, d_out_dist,
-                                      d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset));
+                                      d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset, nullptr, 0));
     }
     return SKM_OK;
 }
 
-// The points `d_ids`, whose lists overflowed, searched again from the same seeds with lists that hold every centroid:
-// rows, norms and seeds are gathered into a compact block, the block goes through the same three kernels in chunks
-// that fit the workspace, results are scattered back.  Same candidates, same thresholds, same walk: same results as
-// lists of that length would have given in the first place.
-int redo_with_full_lists(skm_ctx* ctx, const SearchOperands& o, const float* d_x, const uint64_t* d_ids, size_t mo,
+// The points `d_ids`, whose lists overflowed, searched again from the same seeds through rows of partial distances to
+// all centroids: rows, norms and seeds are gathered into a compact block; per chunk that fits the workspace the seed
+// distances, the dense partial distances (the GEMM core with the distance epilogue: the same values as the candidate
+// kernels compute) and the walk whose first test scans the dense row; results are scattered back.  For a point that a
+// quarter of the centroids pass, a dense row costs less than appending and walking that many list entries (measured
+// against a second pass with full-length lists: 121 against 154 ms for the 685,000 overflowing points of an
+// AssignTrainingPoints with the reference's defaults at n = 1M, k = 10,000; 13.1 against 14.5 ms for the 86,000 of the
+// second iteration of a Train), and for a handful of points the GEMM spreads over centroid tiles where a candidate
+// kernel would sweep them with one workgroup.
+int redo_with_dense_rows(skm_ctx* ctx, const SearchOperands& o, const float* d_x, const uint64_t* d_ids, size_t mo,
                          const float* d_xnorm_p, uint32_t* d_inout_idx, float* d_out_dist, uint32_t* d_counts,
                          unsigned long long* stage_arg) {
-    const uint32_t cap = (uint32_t) align_up(o.k, 64);
-    size_t chunk = ctx->workspace_limit / (size_t(cap) * sizeof(uint2));
+    const size_t ld = align_up(o.k, 64);
+    size_t chunk = ctx->workspace_limit / (ld * sizeof(float));
     chunk = std::max<size_t>(128, (chunk / 128) * 128);
+    chunk = std::min<size_t>(chunk, size_t(1) << 22);
     chunk = std::min(chunk, align_up(mo, 128));
     const size_t mo_pad = align_up(mo, 64);
     void* ws_o = nullptr;
-    SKM_TRY(workspace(ctx, 3, mo * o.d * sizeof(float) + (8 * mo_pad + 64) * sizeof(uint32_t) + mo_pad * sizeof(uint64_t), &ws_o));
-    uint64_t* over2 = (uint64_t*) ws_o;  // never filled: no list overflows
-    float* xo = (float*) (over2 + mo_pad);
+    SKM_TRY(workspace(ctx, 3, mo * o.d * sizeof(float) + 6 * mo_pad * sizeof(uint32_t), &ws_o));
+    float* xo = (float*) ws_o;
     float* xnorm_o = xo + mo * o.d;
     uint32_t* idx_o = (uint32_t*) (xnorm_o + mo_pad);
     float* dist_o = (float*) (idx_o + mo_pad);
     uint32_t* cnt_o = (uint32_t*) (dist_o + mo_pad);
     float* best0_o = (float*) (cnt_o + mo_pad);
     float* thr0_o = best0_o + mo_pad;
-    uint32_t* cand_count_o = (uint32_t*) (thr0_o + mo_pad);
-    uint32_t* cursor_o = cand_count_o + mo_pad;
-    uint32_t* n_over2 = cursor_o + mo_pad;  // stays 0
     SKM_TRY(skm_gather_rows(ctx, d_x, o.d, d_ids, mo, xo, d_xnorm_p, xnorm_o));
     SKM_TRY(launch_gather_u32(ctx, d_inout_idx, d_ids, (int) mo, idx_o));
+    void* ws_partial = nullptr;
+    SKM_TRY(workspace(ctx, 0, std::min(chunk, mo) * ld * sizeof(float), &ws_partial));
     for (size_t i0 = 0; i0 < mo; i0 += chunk) {
         const size_t m = std::min(chunk, mo - i0);
-        void* ws_cand = nullptr;
-        SKM_TRY(workspace(ctx, 0, m * size_t(cap) * sizeof(uint2), &ws_cand));
-        SKM_TRY(search_chunk(ctx, o, xo + i0 * o.d, m, xnorm_o + i0, cap, (uint2*) ws_cand, best0_o + i0, thr0_o + i0,
-                             cand_count_o + i0, idx_o + i0, dist_o + i0, cnt_o + i0, stage_arg, nullptr, over2, n_over2, i0,
-                             i0 == 0, true, cursor_o + i0, "search/overflow/seed", "search/overflow/blas", "search/overflow/pdx"));
+        {
+            ScopedStage st(ctx, "search/overflow/seed");
+            SKM_TRY(launch_seed_distance(ctx, xo + i0 * o.d, o.d_c, idx_o + i0, (int) m, (int) o.d, o.d_ratios,
+                                         (int) o.partial_d, best0_o + i0, thr0_o + i0, nullptr, nullptr));
+        }
+        {
+            ScopedStage st(ctx, "search/overflow/blas");
+            SKM_TRY(launch_gemm_store(ctx, xo + i0 * o.d, (int) m, (int64_t) o.d, o.d_c, (int) o.k, (int64_t) o.d,
+                                      (int) o.partial_d, (float*) ws_partial, (int64_t) ld, xnorm_o + i0, o.d_cnorm_p));
+        }
+        {
+            ScopedStage st(ctx, "search/overflow/pdx");
+            SKM_TRY(launch_prune_list(ctx, nullptr, nullptr, 0, best0_o + i0, xo + i0 * o.d, (int) m, o.d_pdx, o.d_aux,
+                                      (int) o.k, (int) o.d, (int) o.vertical_d, (int) o.partial_d, o.d_ratios, idx_o + i0,
+                                      dist_o + i0, cnt_o + i0, stage_arg, nullptr, nullptr, nullptr, 0,
+                                      (const float*) ws_partial, (int64_t) ld));
+        }
     }
     SKM_TRY(launch_scatter_u32(ctx, idx_o, d_ids, (int) mo, d_inout_idx));
     SKM_TRY(launch_scatter_u32(ctx, (const uint32_t*) dist_o, d_ids, (int) mo, (uint32_t*) d_out_dist));
@@ -180,10 +196,10 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
         SKM_TRY(workspace(ctx, 0, m * size_t(cap) * sizeof(uint2), &ws_cand));
         SKM_TRY(search_chunk(ctx, o, d_x + i0 * d, m, d_xnorm_p + i0, cap, (uint2*) ws_cand, d_best0, d_thr0, d_cand_count,
                              d_inout_idx + i0, d_out_dist + i0, d_counts + i0, stage_arg, order, d_over_ids, d_n_over,
-                             (uint64_t) i0, i0 == 0, false, d_cursor + i0, "search/seed", "search/blas", "search/pdx"));
+                             (uint64_t) i0, i0 == 0, d_cursor + i0));
     }
-    // Points whose list overflowed (loose seeds, or points with no centroid nearby) are searched again with lists that
-    // hold every centroid.  The sum of the
+    // Points whose list overflowed (loose seeds, or points with no centroid nearby) are searched again through dense
+    // rows of partial distances.  The sum of the
     // per-point counts is queued before the number of overflowing points is known and both arrive with one wait;
     // it is taken again only if a redo changed some counts.
     double* h_not_pruned = nullptr;
@@ -197,9 +213,10 @@ extern "C" int skm_assign_pruned(skm_ctx* ctx, const float* d_x, size_t n, const
     }
     SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
     const size_t mo = *(volatile uint32_t*) h_n_over;
+    ctx->last_overflow_points = mo;
     if (mo > 0) {
         ScopedStage st(ctx, "search/overflow");
-        SKM_TRY(redo_with_full_lists(ctx, o, d_x, d_over_ids, mo, d_xnorm_p, d_inout_idx, d_out_dist, d_counts, stage_arg));
+        SKM_TRY(redo_with_dense_rows(ctx, o, d_x, d_over_ids, mo, d_xnorm_p, d_inout_idx, d_out_dist, d_counts, stage_arg));
     }
     if (h_out_not_pruned) {
         double total = *(volatile double*) h_not_pruned;

@@ -155,7 +155,7 @@ def test_both_list_walks_give_the_same_bits(capi, ctx, oracle, blobs, n, d, k, p
 
 def test_both_list_walks_with_loose_ratios(capi, ctx, oracle, blobs):
     """Loose ratios: nearly every candidate survives many blocks, pools fill up (rounds over whole points, a point
-    alone filling most of a pool) and most lists overflow into the pass with full-length lists."""
+    alone filling most of a pool) and most lists overflow into the pass over dense rows."""
     n, d, k = 3000, 256, 2600
     X, C, _ = _setup(oracle, blobs, n, d, k, seed=11)
     prev = np.random.default_rng(3).integers(0, k, n).astype(np.uint32)
@@ -176,7 +176,7 @@ def test_both_list_walks_with_loose_ratios(capi, ctx, oracle, blobs):
 
 def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs):
     """Random seeds at k > 1024: thresholds are loose, many points collect more candidates than their list holds
-    (cap = 1024 slots) and are searched again with full-length lists; the two kernels must still agree bit for bit."""
+    (cap = 1024 slots) and are searched again through dense rows; the two kernels must still agree bit for bit."""
     n, d, k = 3000, 256, 2600
     X, C, _ = _setup(oracle, blobs, n, d, k, seed=11)
     prev = np.random.default_rng(3).integers(0, k, n).astype(np.uint32)

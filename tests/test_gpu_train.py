@@ -364,6 +364,92 @@ def test_hierarchical_train_matches_oracle(capi, ctx, oracle, blobs, n, d, k):
     km.close()
 
 
+@pytest.mark.parametrize("n,d,k,spread", [(40000, 128, 400, 60), (60000, 256, 900, 200), (50000, 256, 2500, 100)])
+def test_hierarchical_decisions_match_the_oracle_iteration_by_iteration(capi, ctx, oracle, blobs, n, d, k, spread):
+    """Decision level of the hierarchical driver (hierarchical_superkmeans.h:262-286,300-420,579-678): for every
+    iteration of every phase the same kind (exact or pruned), the same d' and the same number of SplitClusters edits
+    (re-seeded empty clusters plus balancing pulls: thresholds, weights and RNG acceptance all feed that count), and
+    the same number of iterations per mesocluster, which fixes ArrangeFineClusters' allocation and the mesocluster
+    sizes it was computed from.  The first fine iteration of every mesocluster starts from a state that is the same on
+    both sides (same members in the same order, same Forgy draws): its objective must agree to 1e-4; later
+    iterations to 1e-3 (one near tie resolved the other way moves a centroid of a cluster of a few dozen points)."""
+    X = blobs(n, d, spread, std=0.3, seed=k + 1)
+    cfg = dict(suppress_warnings=1, early_termination=0, iters_refinement=1)
+    km = capi.KMeans(k, d, hierarchical=True, **cfg)
+    ok = oracle.KMeans(k, d, hierarchical=True, **cfg)
+    C, OC = km.train(X), ok.train(X)
+    for which in (1, 2):
+        gs, os_ = km.stats(which), ok.stats(which)
+        assert [(a.iteration, bool(a.is_gemm_only), a.partial_d) for a in gs] == \
+               [(b.iteration, bool(b.is_gemm_only), b.partial_d) for b in os_], f"phase {which}"
+        if which == 1 or n // k >= 60:
+            assert [a.split for a in gs] == [b.split for b in os_], f"phase {which}"
+        else:
+            # twenty points per cluster: one point assigned the other way changes a size that the balancing rule
+            # compares with a threshold of five.  Exact where the state is still the same (first iteration of every
+            # mesocluster), in aggregate afterwards.
+            first_it = gs[0].iteration
+            assert [a.split for a in gs if a.iteration == first_it] == [b.split for b in os_ if b.iteration == first_it]
+            assert abs(sum(a.split for a in gs) - sum(b.split for b in os_)) <= 0.05 * sum(b.split for b in os_)
+    # the refinement starts from the fine phase's end state, where a handful of points sit in different clusters: a
+    # size next to the balancing threshold then falls on the other side of it
+    gs, os_ = km.stats(3), ok.stats(3)
+    assert [(a.iteration, bool(a.is_gemm_only), a.partial_d) for a in gs] == \
+           [(b.iteration, bool(b.is_gemm_only), b.partial_d) for b in os_]
+    for a, b in zip(gs, os_):
+        assert abs(int(a.split) - int(b.split)) <= max(2, 0.1 * b.split)
+        assert abs(a.objective - b.objective_f64) <= 2e-3 * b.objective_f64
+    gs, os_ = km.stats(2), ok.stats(2)
+    firsts = [i for i, s in enumerate(gs) if s.iteration == gs[0].iteration]
+    assert len(firsts) == int(round(np.sqrt(k)))  # every mesocluster was clustered
+    assert any(s.split > 0 for s in gs)  # the balancing step did decide something on this data
+    for i, (a, b) in enumerate(zip(gs, os_)):
+        bar = 1e-4 if i in firsts else (1e-3 if n // k >= 60 else 2e-2)
+        assert abs(a.objective - b.objective_f64) <= bar * max(b.objective_f64, 1e-9), f"fine iteration {i}"
+        if not a.is_gemm_only:
+            assert abs(a.not_pruned_pct - b.not_pruned_pct) <= 2e-2 * max(b.not_pruned_pct, 1e-6) + 1e-6
+    ga = km.assignments(n)
+    _, oa, _, osizes = ok.state()
+    assert np.mean(ga != oa) <= (5e-3 if n // k >= 60 else 0.2)
+    km.close()
+
+
+def test_hierarchical_with_a_mesocluster_emptied_in_the_last_meso_iteration(capi, ctx, oracle, blobs):
+    """Where this driver departs from the reference on purpose.  A third of the rows are copies of one vector, so two
+    of the initial mesocluster centroids coincide and the later one of them gets no point; with one mesoclustering
+    iteration that is the last search before the partition.  SplitClusters re-seeds it and edits cluster_sizes (half
+    the donor's size moves to the empty cluster), and the reference partitions the points by those edited sizes
+    (hierarchical_superkmeans.h:262-286), which no longer match the assignments it compacts by: its fine clusterings
+    then read members past the end of a mesocluster's range (the oracle, which follows the reference there, aborts
+    on this input, so it is not run).  Here the sizes are recounted from the assignments: the emptied mesocluster has
+    no members and receives no fine clusters, and the result must be a consistent clustering: fewer fine
+    clusterings than mesoclusters, the copies of one vector in one cluster, and a WCSS of the returned assignments in
+    the range of what a flat k-means of the same k reaches."""
+    n, d, k = 6000, 128, 144
+    X = blobs(n, d, 40, std=0.3, seed=5)
+    X[::3] = X[0]
+    cfg = dict(suppress_warnings=1, early_termination=0, iters_mesoclustering=1, iters_refinement=0)
+    km = capi.KMeans(k, d, hierarchical=True, **cfg)
+    C = km.train(X)
+    gm = km.stats(1)
+    assert len(gm) == 1 and gm[0].is_gemm_only
+    assert gm[0].split >= 1  # premise: a mesocluster was empty and re-seeded in the last (only) meso iteration
+    n_meso = int(round(np.sqrt(k)))
+    gf = km.stats(2)
+    starts = [i for i, s in enumerate(gf) if s.iteration == gf[0].iteration]
+    assert 1 <= len(starts) < n_meso  # emptied mesoclusters were not clustered
+    ga = km.assignments(n)
+    assert ga.max() < k
+    assert len(np.unique(ga[::3])) == 1  # the copies of one vector are one point
+    # quality of the returned assignments against the returned centroids: in the range of a flat k-means of the same k
+    wcss = ((X.astype(np.float64) - C[ga].astype(np.float64)) ** 2).sum()
+    flat = capi.KMeans(k, d, iters=3, sampling_fraction=1.0, early_termination=0, suppress_warnings=1)
+    flat.train(X)
+    assert wcss <= 1.5 * flat.stats()[-1].objective
+    flat.close()
+    km.close()
+
+
 def test_hierarchical_results_do_not_depend_on_the_number_of_helpers(capi, ctx, blobs):
     """The fine clusterings of the mesoclusters run on n_threads helper objects (own stream, own scratch) that write
     disjoint ranges of the owner's buffers.  Every problem is computed as it would be alone, so 1, 8 and 12 helpers
