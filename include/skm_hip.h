@@ -62,9 +62,10 @@ int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
 int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which);
 
 /* Which kernel walks the candidate lists of skm_assign_pruned (tuning and test knob; results do not depend on it):
- * 0 = automatic (default: eight points pooled per wavefront for calls of at least 32,768 points whose rows are 16-byte
- * aligned with d a multiple of 4, except for the second pass over points whose lists overflowed; one point per
- * wavefront otherwise), 1 = always one point per wavefront, 2 = pooled wherever the rows allow it. */
+ * 0 = automatic (default: several points pooled per wavefront for calls of at least 32,768 points whose rows are
+ * 16-byte aligned with d a multiple of 4, eight points from 500,000 points on and four below; one point per wavefront
+ * otherwise), 1 = always one point per wavefront, 2 / 3 = pooled with four / eight points per wavefront wherever the
+ * rows allow it.  The second pass over points whose list overflowed always takes one point per wavefront. */
 int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which);
 /* Into how many launches the pooled walk of a call is split, each over a contiguous range of the batches of 1024
  * centroids, all points walking one range before any walks the next (default 1; capped at the number of batches;

@@ -1,4 +1,4 @@
-// Pruned search over per-point candidate lists, POOL_PTS points per wavefront.
+// Pruned search over per-point candidate lists, several points (POOL_PTS: 4 or 8) per wavefront.
 //
 // Same contract and same arithmetic as prune_list_kernel (kernels_prune.hip): for every point the batches of 1024
 // centroids are taken in ascending order, the candidates of a batch meet the threshold best * ratios[d'] and then
@@ -25,13 +25,19 @@
 
 namespace skm {
 
-constexpr int POOL_PTS = 8;                   // points per wavefront
+// Points per wavefront: 8 where the call has points enough to fill the chip many times over, 4 below (the chain of
+// dependent steps of a batch is shorter and there are twice as many wavefronts; measured on the walks of a whole
+// Train: 2,000,000 points 216 ms with 8 and 233 ms with 4, 1,000,000 points 15.5 and 16.0 ms, 100,000 points 5.3 and
+// 4.0 ms; 16 points per wavefront lose everywhere).
+constexpr int POOL_PTS_MANY = 8, POOL_PTS_FEW = 4;
+constexpr int POOL_MANY_POINTS = 500000;
 constexpr int POOL_CAP = SKM_Y_BATCH_SIZE;    // pool entries: one whole batch of one point always fits
 constexpr int POOL_NONE = 0x7fffffff;
 constexpr int POOL_Q_SHIFT = 10;              // entry key = point slot << 10 | position in the batch
 constexpr uint32_t POOL_POS_MASK = SKM_Y_BATCH_SIZE - 1;
 static_assert(SKM_Y_BATCH_SIZE == 1024 && SKM_H_DIM_SIZE == 64, "key layout and block addressing assume 1024 x 64");
 
+template <int POOL_PTS>
 struct __attribute__((aligned(16))) PoolLds {  // per wavefront
     float xs[POOL_PTS * SKM_H_DIM_SIZE];   // slices of the points' rows for the current block
     float acc[POOL_CAP + LIST_PAD];
@@ -58,7 +64,8 @@ __device__ __forceinline__ float readlane_f(float v, int l) {
 }
 
 // Keeps the entries below their point's threshold (L.thr), preserving order; in place (see compact_survivors).
-__device__ __forceinline__ int pool_compact(PoolLds& L, int cnt, int lane) {
+template <class Lds>
+__device__ __forceinline__ int pool_compact(Lds& L, int cnt, int lane) {
     int out = 0;
     for (int s0 = 0; s0 < cnt; s0 += 64) {
         const int s = s0 + lane;
@@ -81,7 +88,8 @@ __device__ __forceinline__ int pool_compact(PoolLds& L, int cnt, int lane) {
 // it, the point's best candidate stays what it is.  A point's entries are contiguous, so "only one" is read off the
 // neighbours' tags.  In place: slot s0 - 1, which the first lane of a later round of the loop reads, is rewritten by
 // the round before only with the entry it already holds.
-__device__ __forceinline__ int pool_drop_lone_incumbents(PoolLds& L, int cnt, int lane) {
+template <class Lds>
+__device__ __forceinline__ int pool_drop_lone_incumbents(Lds& L, int cnt, int lane) {
     int out = 0;
     for (int s0 = 0; s0 < cnt; s0 += 64) {
         const int s = s0 + lane;
@@ -104,12 +112,15 @@ __device__ __forceinline__ int pool_drop_lone_incumbents(PoolLds& L, int cnt, in
     return out;
 }
 
-template <bool ACCT>  // ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking)
+// ACCT: per-step pair counts requested (adds atomics and keeps lone incumbents walking).  POOL_PTS: points per
+// wavefront, 4 or 8.
+template <bool ACCT, int POOL_PTS>
 __global__ __launch_bounds__(PRUNE_WAVES * 64, 4) void prune_pool_kernel(PruneListArgs a) {
-    __shared__ PoolLds s_all[PRUNE_WAVES];
+    constexpr int POOL_XL = POOL_PTS / 4;  // slices a lane stages per block
+    __shared__ PoolLds<POOL_PTS> s_all[PRUNE_WAVES];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    PoolLds& L = s_all[wave];
+    PoolLds<POOL_PTS>& L = s_all[wave];
     const int sub = lane & 15, grp = lane >> 4;
     // consecutive slots of the visiting order stay on one compute die (see point_of_wave)
     const int per_die = (int) (gridDim.x / 8);
@@ -171,9 +182,8 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 4) void prune_pool_kernel(PruneLi
             nextb = (lane == q && cursor < ncand) ? (int) (first / SKM_Y_BATCH_SIZE) : nextb;
         }
         int jb = nextb;
-        jb = min(jb, __shfl_xor(jb, 1));
-        jb = min(jb, __shfl_xor(jb, 2));
-        jb = min(jb, __shfl_xor(jb, 4));
+#pragma unroll
+        for (int off = 1; off < POOL_PTS; off <<= 1) jb = min(jb, __shfl_xor(jb, off));
         jb = __builtin_amdgcn_readfirstlane(jb);
         if (jb >= a.jb_hi) break;  // POOL_NONE: no entry left
         const int base = jb * SKM_Y_BATCH_SIZE;
@@ -248,14 +258,17 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 4) void prune_pool_kernel(PruneLi
             q_start = q_stop;
             if (cnt == 0) continue;
 
-            // rows whose slices are staged: lanes of group g serve point slots g and g + 4; a slot that contributed
+            // rows whose slices are staged: lanes of group g serve point slots g, g + 4, ...; a slot that contributed
             // nothing to this round reads the row of one that did
             const int q_any = __builtin_ctz(contrib);
-            const int qa = ((contrib >> grp) & 1u) ? grp : q_any;
-            const int qb = ((contrib >> (grp + 4)) & 1u) ? grp + 4 : q_any;
-            const float* xrow_a = a.x + (int64_t) L.pid[qa] * d + V + sub * 4;
-            const float* xrow_b = a.x + (int64_t) L.pid[qb] * d + V + sub * 4;
-            float4 xa = make_float4(0.0f, 0.0f, 0.0f, 0.0f), xb = xa;
+            const float* xrow[POOL_XL];
+            float4 xnext[POOL_XL];
+#pragma unroll
+            for (int j = 0; j < POOL_XL; ++j) {
+                const int qj = ((contrib >> (grp + 4 * j)) & 1u) ? grp + 4 * j : q_any;
+                xrow[j] = a.x + (int64_t) L.pid[qj] * d + V + sub * 4;
+                xnext[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
             bool staged = false;
 
             // ---- horizontal blocks of 64 dimensions, PDX layout (pdxearch.h:149-180) ----
@@ -320,15 +333,17 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 4) void prune_pool_kernel(PruneLi
                     if (ACCT && lane == 0) atomicAdd(&acct[1 + hb], (unsigned long long) cnt);
                     // this block's slices were requested one block ago; the next ones are requested now
                     if (!staged) {
-                        xa = *reinterpret_cast<const float4*>(xrow_a + hb * SKM_H_DIM_SIZE);
-                        xb = *reinterpret_cast<const float4*>(xrow_b + hb * SKM_H_DIM_SIZE);
+#pragma unroll
+                        for (int j = 0; j < POOL_XL; ++j) xnext[j] = *reinterpret_cast<const float4*>(xrow[j] + hb * SKM_H_DIM_SIZE);
                         staged = true;
                     }
-                    *reinterpret_cast<float4*>(&L.xs[grp * SKM_H_DIM_SIZE + sub * 4]) = xa;
-                    *reinterpret_cast<float4*>(&L.xs[(grp + 4) * SKM_H_DIM_SIZE + sub * 4]) = xb;
+#pragma unroll
+                    for (int j = 0; j < POOL_XL; ++j)
+                        *reinterpret_cast<float4*>(&L.xs[(grp + 4 * j) * SKM_H_DIM_SIZE + sub * 4]) = xnext[j];
                     if (hb + 1 < n_hblocks) {
-                        xa = *reinterpret_cast<const float4*>(xrow_a + (hb + 1) * SKM_H_DIM_SIZE);
-                        xb = *reinterpret_cast<const float4*>(xrow_b + (hb + 1) * SKM_H_DIM_SIZE);
+#pragma unroll
+                        for (int j = 0; j < POOL_XL; ++j)
+                            xnext[j] = *reinterpret_cast<const float4*>(xrow[j] + (hb + 1) * SKM_H_DIM_SIZE);
                     }
                     // 32 entries per pass: the eight gathers of a lane are issued before any of them is used.  Slots
                     // past the last entry read the pad (key 0) and their sums land in the pad.
@@ -439,8 +454,10 @@ int launch_prune_pool(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
-                      uint64_t id_offset, int jb_lo, int jb_hi, uint32_t* cursor) {
+                      uint64_t id_offset, int jb_lo, int jb_hi, uint32_t* cursor, int points_per_wavefront) {
     if (n_chunk <= 0) return SKM_OK;
+    if (points_per_wavefront != 0 && points_per_wavefront != POOL_PTS_FEW && points_per_wavefront != POOL_PTS_MANY)
+        return set_error(SKM_ERR_INVALID, "pooled list walk: 4 or 8 points per wavefront");
     if (jb_lo < 0 || jb_hi <= jb_lo || ((jb_lo > 0 || jb_hi < (k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE) && !cursor))
         return set_error(SKM_ERR_INVALID, "pooled list walk: a range of batches needs the cursor array");
     if (!prune_pool_serves(x, pdx, d))
@@ -453,12 +470,18 @@ int launch_prune_pool(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
     a.n = n_chunk; a.k = k; a.d = d; a.vertical_d = vertical_d; a.partial_d = partial_d;
     a.jb_lo = jb_lo; a.jb_hi = jb_hi; a.cursor = cursor;
     a.partial = nullptr; a.ld_partial = 0;
-    const int wavefronts = (n_chunk + POOL_PTS - 1) / POOL_PTS;
+    const int pts = points_per_wavefront ? points_per_wavefront
+                                         : (n_chunk >= POOL_MANY_POINTS ? POOL_PTS_MANY : POOL_PTS_FEW);
+    const int wavefronts = (n_chunk + pts - 1) / pts;
     dim3 grid(die_striped_groups(wavefronts, PRUNE_WAVES)), block(PRUNE_WAVES * 64);
-    if (d_stage_pairs)
-        hipLaunchKernelGGL((prune_pool_kernel<true>), grid, block, 0, ctx->stream, a);
+    if (d_stage_pairs && pts == POOL_PTS_MANY)
+        hipLaunchKernelGGL((prune_pool_kernel<true, POOL_PTS_MANY>), grid, block, 0, ctx->stream, a);
+    else if (d_stage_pairs)
+        hipLaunchKernelGGL((prune_pool_kernel<true, POOL_PTS_FEW>), grid, block, 0, ctx->stream, a);
+    else if (pts == POOL_PTS_MANY)
+        hipLaunchKernelGGL((prune_pool_kernel<false, POOL_PTS_MANY>), grid, block, 0, ctx->stream, a);
     else
-        hipLaunchKernelGGL((prune_pool_kernel<false>), grid, block, 0, ctx->stream, a);
+        hipLaunchKernelGGL((prune_pool_kernel<false, POOL_PTS_FEW>), grid, block, 0, ctx->stream, a);
     return check_hip(hipGetLastError(), "prune_pool_kernel launch");
 }
 

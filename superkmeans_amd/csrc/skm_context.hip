@@ -343,7 +343,7 @@ int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which) {
 
 int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which) {
     SKM_REQUIRE(ctx, "null context");
-    SKM_REQUIRE(which >= 0 && which <= 2, "which must be 0 (automatic), 1 (one point per wavefront) or 2 (pooled)");
+    SKM_REQUIRE(which >= 0 && which <= 3, "which must be 0 (automatic), 1 (one point per wavefront), 2 or 3 (pooled, 4 or 8 points)");
     ctx->walk_kernel = which;
     return SKM_OK;
 }

@@ -158,13 +158,14 @@ int launch_prune_list(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_coun
                       uint64_t id_offset, const float* dense_partial, int64_t ld_partial);
 // The same walk with several points per wavefront (rows 16-byte aligned, d a multiple of 4); `serves` says whether a
 // call qualifies.  Same results bit for bit.  One launch walks the batches [jb_lo, jb_hi) of 1024 centroids; a walk
-// split over several launches (ascending ranges) keeps its place in `cursor` (n_chunk words).
+// split over several launches (ascending ranges) keeps its place in `cursor` (n_chunk words).  points_per_wavefront: 4, 8,
+// or 0 for the choice by the number of points.
 bool prune_pool_serves(const float* x, const float* pdx, int d);
 int launch_prune_pool(skm_ctx* ctx, const uint2* cand, const uint32_t* cand_count, uint32_t cap, const float* best0,
                       const float* x, int n_chunk, const float* pdx, const float* aux, int k, int d, int vertical_d,
                       int partial_d, const float* ratios, uint32_t* inout_idx, float* out_dist, uint32_t* out_not_pruned,
                       unsigned long long* d_stage_pairs, const uint32_t* order, uint64_t* over_ids, uint32_t* n_over,
-                      uint64_t id_offset, int jb_lo, int jb_hi, uint32_t* cursor);
+                      uint64_t id_offset, int jb_lo, int jb_hi, uint32_t* cursor, int points_per_wavefront);
 int launch_gather_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 int launch_scatter_u32(skm_ctx* ctx, const uint32_t* in, const uint64_t* ids, int m, uint32_t* out);
 

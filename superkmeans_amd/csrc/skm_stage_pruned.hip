@@ -64,7 +64,8 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
         // Several points per wavefront pay when the points are many: with few points an eighth as many wavefronts
         // do not fill the chip.
         const bool pooled = ctx->walk_kernel != 1 && prune_pool_serves(xc, o.d_pdx, (int) o.d) &&
-                            (ctx->walk_kernel == 2 || m >= 32768);
+                            (ctx->walk_kernel >= 2 || m >= 32768);
+        const int points_per_wavefront = ctx->walk_kernel == 2 ? 4 : (ctx->walk_kernel == 3 ? 8 : 0);
         if (pooled) {
             const int n_batches = (int) ((o.k + SKM_Y_BATCH_SIZE - 1) / SKM_Y_BATCH_SIZE);
             const int phases = std::max(1, std::min(ctx->walk_launches, n_batches));
@@ -72,7 +73,8 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
                 const int lo = (int) ((int64_t) n_batches * ph / phases), hi = (int) ((int64_t) n_batches * (ph + 1) / phases);
                 SKM_TRY(launch_prune_pool(ctx, d_cand, d_cand_count, cap, d_best0, xc, (int) m, o.d_pdx, o.d_aux, (int) o.k,
                                           (int) o.d, (int) o.vertical_d, (int) o.partial_d, o.d_ratios, d_inout_idx, d_out_dist,
-                                          d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset, lo, hi, d_cursor));
+                                          d_counts, stage_arg, order, d_over_ids, d_n_over, id_offset, lo, hi, d_cursor,
+                                          points_per_wavefront));
             }
         } else
             SKM_TRY(launch_prune_list(ctx, d_cand, d_cand_count, cap, d_best0, xc, (int) m, o.d_pdx, o.d_aux, (int) o.k,

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, kernel=0, walk=0, launches=1):
     """kernel: skm_ctx_set_candidate_kernel (0 automatic, 1 tiled, 2 register-stationary where the shape allows);
-    walk: skm_ctx_set_walk_kernel (0 automatic, 1 one point per wavefront, 2 pooled wherever rows are aligned)."""
+    walk: skm_ctx_set_walk_kernel (0 automatic, 1 one point per wavefront, 2 / 3 four / eight points pooled per wavefront)."""
     n, d = X.shape
     k = C.shape[0]
     H, V = oracle.dimension_split(d)
@@ -145,11 +145,12 @@ def test_both_list_walks_give_the_same_bits(capi, ctx, oracle, blobs, n, d, k, p
         prev = np.random.default_rng(n).integers(0, k, n).astype(np.uint32)
     ratios = oracle.ratios(d, 1.5)
     single = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=1)
-    pooled = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=2)
-    _same_bits(single, pooled)
+    for walk in (2, 3):
+        pooled = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=walk)
+        _same_bits(single, pooled)
     # the pooled walk split into one launch per batch, or per range of batches, resumes from the state the launch before left
-    for launches in (2, 1000):
-        split = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=2, launches=launches)
+    for walk, launches in ((2, 2), (3, 1000)):
+        split = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, walk=walk, launches=launches)
         _same_bits(single, split)
 
 
@@ -163,12 +164,14 @@ def test_both_list_walks_with_loose_ratios(capi, ctx, oracle, blobs):
     ratios[d] = 1.0
     for accounting in (False, True):
         single = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, accounting=accounting, walk=1)
-        pooled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, accounting=accounting, walk=2)
-        _same_bits(single, pooled)
+        for walk in (2, 3):
+            pooled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, accounting=accounting, walk=walk)
+            _same_bits(single, pooled)
     ones = np.ones(d + 1, dtype=np.float32)  # nothing is ever pruned: every pool is as full as it can get
     single = _pruned(capi, ctx, oracle, X[:600], C, prev[:600], 40, ones, accounting=True, walk=1)
-    pooled = _pruned(capi, ctx, oracle, X[:600], C, prev[:600], 40, ones, accounting=True, walk=2)
-    _same_bits(single, pooled)
+    for walk in (2, 3):
+        pooled = _pruned(capi, ctx, oracle, X[:600], C, prev[:600], 40, ones, accounting=True, walk=walk)
+        _same_bits(single, pooled)
     bi, bbest, bsecond = oracle.brute_force(X[:600], C)
     tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
     assert np.all((pooled[0] == bi) | tie)
