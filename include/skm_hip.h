@@ -57,8 +57,9 @@ int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes);
 
 /* Which kernel computes the partial distances of skm_assign_pruned (tuning and test knob; results do not depend on
  * it): 0 = automatic (default: the register-stationary kernel for partial_d <= 160 and at least 49,152 points per
- * call, the tiled 128 x 128 kernel otherwise), 1 = always the tiled kernel, 2 = the register-stationary kernel
- * whenever partial_d <= 160 and the rows are 16-byte aligned, whatever the number of points. */
+ * call, the kernel with 256 x 256 tiles for partial_d > 160 and at least 49,152 points, the tiled 128 x 128 kernel
+ * otherwise), 1 = always the 128 x 128 kernel, 2 = the register-stationary kernel whenever partial_d <= 160 and the rows
+ * are 16-byte aligned, whatever the number of points, 3 = always the 256 x 256 kernel. */
 int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which);
 
 /* Which kernel walks the candidate lists of skm_assign_pruned (tuning and test knob; results do not depend on it):

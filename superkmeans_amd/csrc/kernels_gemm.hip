@@ -573,11 +573,123 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_candidates_kernel(
     if (tid < GEMM_TN && tn * GEMM_TN + tid < g.N) cand_count[tn * GEMM_TN + tid] = cnt_s[tid];
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same contract for long d' (from about 160 leading dimensions on): a tile is then many operand slices long, the
+// per-tile prologue is a few per cent of the tile, and what counts is the main loop.  A workgroup of the large shape
+// (8 wavefronts of 128 x 64, one per CU) owns 256 points and sweeps the 256-centroid tiles in ascending order (a batch
+// of 1024 centroids is four consecutive tiles, so a point's candidates are still appended batch after batch) with the
+// tile loop of the GEMM core: per MFMA half the global loads, LDS stores and barriers of the 128 x 128 shape.  The
+// epilogue is gemm_candidates_kernel's on 4 x 2 accumulator blocks: the norms of the tile's centroids come from LDS
+// (two slots: tile t + 1 writes the slot tile t - 1 read, and every wavefront has passed a barrier of tile t's loop in
+// between), the 64 tests of a point are shifted into two bit masks, lanes with a bit append.  Products are accumulated
+// in the order of every other shape, so the emitted pairs carry the same bits.
+// ---------------------------------------------------------------------------------------------
+template <bool VEC>
+__global__ __launch_bounds__(GemmBig::THREADS, 1) void gemm_candidates_big_kernel(
+    GemmOperands g, const float* __restrict__ xnorm, const float* __restrict__ cnorm,
+    const float* __restrict__ thr0, uint32_t* __restrict__ cand_count, uint2* __restrict__ cand, uint32_t cap
+) {
+    using S = GemmBig;
+    extern __shared__ float lds[];
+    float* cn_s = lds + S::LDS_FLOATS;                                      // [2][TM]
+    uint32_t* cnt_s = reinterpret_cast<uint32_t*>(cn_s + 2 * S::TM);        // [TN]
+    const int tn = blockIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / S::WN, wn = wave % S::WN;
+
+    // |x|^2 and the threshold of the workgroup's points wait in LDS for the epilogues: held in registers across the
+    // tile loop they would not fit next to its 128 accumulators
+    float2* pt_s = reinterpret_cast<float2*>(cnt_s + S::TN);  // [TN] {|x|^2, threshold}
+    if (tid < S::TN) {
+        const int p = tn * S::TN + tid;
+        const bool valid = p < g.N;
+        pt_s[tid] = make_float2(valid ? xnorm[p] : 0.0f, valid ? thr0[p] : -3.0e38f);  // nothing passes for padding columns
+        cnt_s[tid] = 0u;
+    }
+
+    for (int tm = 0; tm < g.tiles_m; ++tm) {
+        if (tid < S::TM) {
+            const int m = tm * S::TM + tid;
+            cn_s[(tm & 1) * S::TM + tid] = m < g.M ? cnorm[m] : 3.0e38f;  // rows past M never pass
+        }
+        WaveAccT<S::FM, S::FN> acc;
+        gemm_tile<VEC, S>(g, tm, tn, lds, acc);  // its barriers order the norms (and cnt_s) before the epilogue
+
+        const float* cns = cn_s + (tm & 1) * S::TM + wm * S::WAVE_M;
+        const int m0 = tm * S::TM + wm * S::WAVE_M;
+#pragma unroll
+        for (int nb = 0; nb < S::FN; ++nb) {
+            const int col = wn * S::WAVE_N + acc_col(nb, lane);
+            const float2 xt = pt_s[col];
+            const float xn = xt.x, thr = xt.y;
+            uint32_t pass[S::FM / 2];  // element (mb, r) lands in bit 31 - ((mb % 2) * 16 + r) of pass[mb / 2]
+#pragma unroll
+            for (int h = 0; h < S::FM / 2; ++h) pass[h] = 0u;
+#pragma unroll
+            for (int mb = 0; mb < S::FM; ++mb) {
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    const floatx4 c4 = *reinterpret_cast<const floatx4*>(&cns[acc_row(mb, r4 * 4, lane)]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int r = r4 * 4 + j;
+                        const float v = fmaf(-2.0f, acc.v[mb][nb][r], xn) + c4[j];
+                        acc.v[mb][nb][r] = v;
+                        // v < thr  <=>  the IEEE difference v - thr carries a set sign bit.
+                        pass[mb / 2] = __builtin_amdgcn_alignbit(pass[mb / 2], __float_as_uint(v - thr), 31);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // bounds how many norms are held at once
+            }
+            uint32_t any = 0u, total = 0u;
+#pragma unroll
+            for (int h = 0; h < S::FM / 2; ++h) {
+                any |= pass[h];
+                total += (uint32_t) __popc(pass[h]);
+            }
+            if (any) {
+                uint32_t slot = atomicAdd(&cnt_s[col], total);
+                const int p = tn * S::TN + col;  // a padding column has no bit set
+                uint2* const list = cand + (int64_t) p * cap;
+#pragma unroll
+                for (int mb = 0; mb < S::FM; ++mb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        if (pass[mb / 2] & (0x80000000u >> ((mb % 2) * 16 + r))) {
+                            if (slot < cap)
+                                list[slot] = make_uint2((uint32_t) (m0 + acc_row(mb, r, lane)), __float_as_uint(acc.v[mb][nb][r]));
+                            ++slot;
+                        }
+                    }
+            }
+        }
+    }
+    __syncthreads();
+    if (tid < S::TN && tn * S::TN + tid < g.N) cand_count[tn * S::TN + tid] = cnt_s[tid];
+}
+
+// The large shape serves long d' on enough points to fill the chip with 256-point workgroups.
+constexpr int CANDIDATES_BIG_MIN_D = 161;
+constexpr int CANDIDATES_BIG_MIN_POINTS = 192 * GemmBig::TN;
+
 int launch_gemm_candidates(skm_ctx* ctx, const float* C, int k, const float* X, int n, int partial_d, int64_t ld,
                            const float* xnorm_p, const float* cnorm_p, const float* thr0, uint32_t* cand_count,
                            uint2* cand, uint32_t cap) {
     if (k <= 0 || n <= 0 || partial_d <= 0) return SKM_OK;
     GemmOperands g;
+    if (ctx->candidate_kernel == 3 ||
+        (partial_d >= CANDIDATES_BIG_MIN_D && n >= CANDIDATES_BIG_MIN_POINTS && ctx->candidate_kernel != 1)) {
+        SKM_TRY(fill_operands<GemmBig>(g, C, k, ld, X, n, ld, partial_d));
+        const size_t lds_bytes = (GemmBig::LDS_FLOATS + 2 * GemmBig::TM + 3 * GemmBig::TN) * sizeof(float);
+        dim3 grid((unsigned) g.tiles_n), block(GemmBig::THREADS);
+        if (gemm_operands_vectorizable(g))
+            SKM_LAUNCH_GEMM((gemm_candidates_big_kernel<true>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
+        else
+            SKM_LAUNCH_GEMM((gemm_candidates_big_kernel<false>), grid, block, lds_bytes, ctx->stream, g, xnorm_p, cnorm_p, thr0, cand_count, cand, cap);
+        return check_hip(hipGetLastError(), "gemm_candidates_big_kernel launch");
+    }
     SKM_TRY(fill_operands<GemmSmall>(g, C, k, ld, X, n, ld, partial_d));
     const size_t lds_bytes = (GEMM_LDS_FLOATS + 3 * GEMM_TM + GEMM_TN) * sizeof(float);
     dim3 grid((unsigned) g.tiles_n), block(GEMM_THREADS);

@@ -336,7 +336,7 @@ int skm_ctx_set_workspace_limit(skm_ctx* ctx, size_t bytes) {
 
 int skm_ctx_set_candidate_kernel(skm_ctx* ctx, int which) {
     SKM_REQUIRE(ctx, "null context");
-    SKM_REQUIRE(which >= 0 && which <= 2, "which must be 0 (automatic), 1 (tiled) or 2 (register-stationary)");
+    SKM_REQUIRE(which >= 0 && which <= 3, "which must be 0 (automatic), 1 (tiled), 2 (register-stationary) or 3 (large tiles)");
     ctx->candidate_kernel = which;
     return SKM_OK;
 }

@@ -50,7 +50,7 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
         ScopedStage st(ctx, "search/blas");
         // the register-stationary kernel addresses the 64 lists of a wavefront with 32-bit byte offsets
         const bool lists_fit = (uint64_t) cap * 64 * sizeof(uint2) < (uint64_t(1) << 32);
-        if (ctx->candidate_kernel != 1 && lists_fit &&
+        if (ctx->candidate_kernel != 1 && ctx->candidate_kernel != 3 && lists_fit &&
             gemm_candidates_stationary_serves(o.d_c, (int) o.k, xc, (int) m, (int) o.partial_d, (int64_t) o.d,
                                               ctx->candidate_kernel == 2))
             SKM_TRY(launch_gemm_candidates_stationary(ctx, o.d_c, (int) o.k, xc, (int) m, (int) o.partial_d, (int64_t) o.d,

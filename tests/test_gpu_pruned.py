@@ -101,7 +101,12 @@ def test_pruned_matches_oracle(capi, ctx, oracle, blobs, n, d, k, partial_d):
                                              (777, 256, 640, 64), (1100, 600, 1030, 77), (1125, 768, 1100, 88),
                                              (1200, 768, 1100, 89), (1300, 768, 1280, 96), (2600, 1024, 2500, 128),
                                              (100, 1024, 60, 103), (1100, 1024, 1088, 160), (300, 1024, 300, 161),
-                                             (131, 512, 63, 72)])
+                                             (131, 512, 63, 72),
+                                             # long d' (the 256 x 256 kernel's range): whole slices, a trailing slice of
+                                             # one to four groups, rows that are not 16-byte aligned, a last tile of
+                                             # a few centroids and of a few points
+                                             (1500, 1536, 1300, 192), (1100, 1536, 1030, 268), (2300, 1536, 2100, 300),
+                                             (800, 1536, 700, 375), (600, 1026, 520, 230), (1100, 2048, 1025, 512)])
 def test_both_candidate_kernels_give_the_same_bits(capi, ctx, oracle, blobs, n, d, k, partial_d):
     X, C, prev = _setup(oracle, blobs, n, d, k, seed=n + d + partial_d)
     ratios = oracle.ratios(d, 1.5)
@@ -111,6 +116,8 @@ def test_both_candidate_kernels_give_the_same_bits(capi, ctx, oracle, blobs, n, 
     assert np.array_equal(tiled[1].view(np.uint32), stationary[1].view(np.uint32))
     assert tiled[2] == stationary[2]
     assert np.array_equal(tiled[3], stationary[3])
+    big = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=True, kernel=3)  # 256 x 256 tiles
+    _same_bits(tiled, big)
     oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, partial_d, ratios)
     bi, bbest, bsecond = oracle.brute_force(X, C)
     tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
@@ -187,9 +194,11 @@ def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs)
     ratios[d] = 1.0
     tiled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=1)
     stationary = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=2)
-    assert np.array_equal(tiled[0], stationary[0])
+    big = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=3)
+    assert np.array_equal(tiled[0], stationary[0]) and np.array_equal(tiled[0], big[0])
     assert np.array_equal(tiled[1].view(np.uint32), stationary[1].view(np.uint32))
-    assert tiled[2] == stationary[2]
+    assert np.array_equal(tiled[1].view(np.uint32), big[1].view(np.uint32))
+    assert tiled[2] == stationary[2] == big[2]
     oi, od, ocounts = oracle.find_nn_pruned(X, C, prev, 40, ratios)
     assert np.mean(stationary[0] == oi) >= 0.9999
 
