@@ -64,17 +64,17 @@ def kernel_sources_hash():
 # copy kernel of known size: FETCH_SIZE x 1.943, WRITE_SIZE x 1.000), per workload shape.  Every entry names the summary it
 # comes from and the kernel_sources_hash() of the tree that was profiled; the figure is reported only while the tree
 # still hashes to that value (otherwise the JSON carries null and the reason), so it cannot outlive the kernels it describes.
-MEASURED_SOURCES_HASH = "unset"
+MEASURED_SOURCES_HASH = "540c08b27822bfa1"
 MEASURED_TRAFFIC_BYTES = {
     # the two gemm_argmin_kernel launches of an Assign pass
-    (1_000_000, 1024, 10_000): (int(((31_605_895 + 2_005_959) * 1.943 + 609_375 + 7_812) * 1024),
+    (1_000_000, 1024, 10_000): (int(((31_581_196 + 2_005_930) * 1.943 + 609_375 + 7_812) * 1024),
                                 "profiles/gemm_argmin_kernel_assign_n1M_d1024_k10k_hbm_traffic.md"),
 }
 # every seed_distance_kernel and list-walk launch of one Train of (n, d, k, iterations)
 MEASURED_PRUNE_TRAFFIC_BYTES = {
-    (1_000_000, 1024, 10_000, 10): (int((48_587_738 * 1.943 + 1_477_281) * 1024),
+    (1_000_000, 1024, 10_000, 10): (int((49_855_367 * 1.943 + 1_759_912) * 1024),
                                     "profiles/gemm_argmin_kernel_assign_n1M_d1024_k10k_hbm_traffic.md"),
-    (2_000_000, 1536, 4_096, 10): (int((843_855_099 * 1.943 + 2_897_329) * 1024),
+    (2_000_000, 1536, 4_096, 10): (int((881_206_545 * 1.943 + 3_441_800) * 1024),
                                    "profiles/train_n2M_d1536_k4096_kernel_stats_list_walk_traffic.md"),
 }
 
@@ -177,9 +177,17 @@ def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps,
     no_train = args.no_train or (train_iters == 0 and not hierarchical)
     if hierarchical:
         cfg = dict(early_termination=0, seed=42, suppress_warnings=1)  # 3 + 5 + 0 iterations, the reference's defaults
+        if args.n_threads is not None:
+            cfg["n_threads"] = args.n_threads
     else:
         cfg = dict(iters=max(1, train_iters), sampling_fraction=1.0, early_termination=0, seed=42, suppress_warnings=1)
-    km = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
+    def new_object():
+        obj = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
+        _capi.check(obj.lib.skm_ctx_set_walk_kernel(obj.ctx.handle, args.walk_kernel))
+        _capi.check(obj.lib.skm_ctx_set_walk_launches(obj.ctx.handle, args.walk_launches))
+        return obj
+
+    km = new_object()
     ctx, lib = km.ctx, km.lib
 
     # ---- synthetic points, resident in HBM ----
@@ -207,7 +215,7 @@ def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps,
         # A second, untimed Train of an identical object only to count the pairs entering each pruning step.
         acct = []
         if n_pruned and not hierarchical:
-            km2 = _capi.KMeans(k, d, **cfg)
+            km2 = new_object()
             km2.set_prune_accounting(True)
             km2.train_device(dX, n)
             acct = km2.prune_accounting()
@@ -216,14 +224,14 @@ def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps,
         # the first touch of fresh device memory).  A third, identical object finds the blocks in the library's
         # per-device cache: its end-to-end time is reported beside the first, and its per-stage device timers (with the
         # event pairs they add around every stage) make the stage table.
-        km3 = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
+        km3 = new_object()
         km3.set_prune_accounting(False)
         t0 = time.perf_counter()
         km3.train_device(dX, n)
         km3.ctx.sync()
         train_warm_s = time.perf_counter() - t0
         km3.close()
-        km4 = _capi.KMeans(k, d, hierarchical=hierarchical, **cfg)
+        km4 = new_object()
         km4.set_prune_accounting(False)
         km4.ctx.prof_enable(True)
         km4.ctx.prof_reset()
@@ -519,6 +527,15 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain row-copy kernel of known size (1 GiB read + 1 GiB write) three times; "
                          "used to scale the FETCH_SIZE / WRITE_SIZE hardware counters")
+    ap.add_argument("--walk-kernel", type=int, default=0,
+                    help="skm_ctx_set_walk_kernel for every Train of the run (0 automatic, 1 one point per wavefront, "
+                         "2 / 3 four / eight points pooled per wavefront); for profiles that compare the walks")
+    ap.add_argument("--walk-launches", type=int, default=1,
+                    help="skm_ctx_set_walk_launches for every Train of the run (the pooled walk split into that many "
+                         "launches over ranges of centroid batches); for the profile that compares one launch with one per batch")
+    ap.add_argument("--n-threads", type=int, default=None,
+                    help="hierarchical configurations: number of mesoclusters fine-clustered concurrently (the config's "
+                         "n_threads; default 8 helper objects with a host thread and a stream each)")
     ap.add_argument("--print-kernel-hash", action="store_true",
                     help="print kernel_sources_hash() of this tree (what MEASURED_SOURCES_HASH must hold) and exit")
     args = ap.parse_args()

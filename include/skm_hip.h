@@ -75,7 +75,7 @@ int skm_ctx_set_walk_kernel(skm_ctx* ctx, int which);
  * more time than the misses did, which the memory-side cache serves: a knob for measuring that trade. */
 int skm_ctx_set_walk_launches(skm_ctx* ctx, int launches);
 /* How many points of the last skm_assign_pruned call on this context collected more candidates than their list holds
- * and went through the second pass with full-length lists (a measure of how loose the seeds were). */
+ * and went through the second pass over dense rows of partial distances (a measure of how loose the seeds were). */
 int skm_ctx_get_last_overflow(skm_ctx* ctx, uint64_t* out_points);
 
 /* Device memory and transfers (stand in for the reference's std::unique_ptr<float[]> buffers,

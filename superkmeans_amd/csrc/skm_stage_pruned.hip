@@ -89,10 +89,10 @@ int search_chunk(skm_ctx* ctx, const SearchOperands& o, const float* xc, size_t 
 // distances, the dense partial distances (the GEMM core with the distance epilogue: the same values as the candidate
 // kernels compute) and the walk whose first test scans the dense row; results are scattered back.  For a point that a
 // quarter of the centroids pass, a dense row costs less than appending and walking that many list entries (measured
-// against a second pass with full-length lists: 121 against 154 ms for the 685,000 overflowing points of an
-// AssignTrainingPoints with the reference's defaults at n = 1M, k = 10,000; 13.1 against 14.5 ms for the 86,000 of the
-// second iteration of a Train), and for a handful of points the GEMM spreads over centroid tiles where a candidate
-// kernel would sweep them with one workgroup.
+// against a second pass of the candidate kernel with lists that hold every centroid: 137 against 154 ms for the
+// 685,000 overflowing points of an AssignTrainingPoints with the reference's defaults at n = 1M, k = 10,000; 12.3
+// against 14.5 ms for the 86,000 of the second iteration of a Train), and for a handful of points the GEMM spreads
+// over centroid tiles where a candidate kernel sweeps them with one workgroup (0.7 ms per iteration).
 int redo_with_dense_rows(skm_ctx* ctx, const SearchOperands& o, const float* d_x, const uint64_t* d_ids, size_t mo,
                          const float* d_xnorm_p, uint32_t* d_inout_idx, float* d_out_dist, uint32_t* d_counts,
                          unsigned long long* stage_arg) {
