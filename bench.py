@@ -169,7 +169,8 @@ def stage_table(n, d, k, ks, hierarchical, stats, acct, prof, V):
     return stage
 
 
-def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps, warmup, with_cpu, with_host, with_extras):
+def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps, warmup, with_cpu, with_host, with_extras,
+               with_agreement=False):
     """One configuration: Train (first and second object of the process, stage table), timed Assign steps, and on
     request the transfer-inclusive leg, the CPU baseline and the headline extras.  Returns the JSON object."""
     from superkmeans_amd import _capi
@@ -267,8 +268,9 @@ def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps,
                                for nm, v in phase_stats.items()}
             train["owner_device_ms"] = round(iter_ms + ms("rotator"), 2)
             train["fine_phase_and_host_s"] = round(train_s - (iter_ms + ms("rotator")) * 1e-3, 4)
-        if with_extras and not hierarchical and n_pruned and len(stats) >= 2:
-            train["pruned_vs_exact_agreement"] = pruned_vs_exact(args, _capi, km, dX, n, d, k, cfg, stats)
+        if (with_extras or with_agreement) and not hierarchical and n_pruned and len(stats) >= 2:
+            train["pruned_vs_exact_agreement"] = pruned_vs_exact(args, _capi, km, dX, n, d, k, cfg, stats,
+                                                                 oracle_sample=with_extras and not args.no_cpu)
 
     if centroids is None and name == "C3":
         # the fixed, seeded centroids of the Assign-only configuration: the generator's own centres
@@ -366,7 +368,7 @@ def run_config(args, name, n, d, k, train_iters, hierarchical, generator, steps,
     return out
 
 
-def pruned_vs_exact(args, _capi, km, dX, n, d, k, cfg, stats):
+def pruned_vs_exact(args, _capi, km, dX, n, d, k, cfg, stats, oracle_sample):
     """How often the last pruned iteration of the Train kept the exact nearest centroid (ADSampling prunes with a
     probabilistic bound).  Train is deterministic: a run with one iteration less gives the rotated centroids and the
     assignments the last iteration started from; the exact search among those centroids is the truth.  The CPU oracle
@@ -391,7 +393,7 @@ def pruned_vs_exact(args, _capi, km, dX, n, d, k, cfg, stats):
     out = {"iteration": int(last.iteration), "partial_d": int(last.partial_d),
            "gpu_pruned_equals_exact": round(float(np.mean(ae == a_last)), 6),
            "points": n}
-    if not args.no_cpu:
+    if oracle_sample:
         from oracle import oracle as O
 
         O.load()
@@ -499,6 +501,7 @@ def compact(result):
             "train_s_end_to_end": t.get("train_s_end_to_end"),
             "train_s_end_to_end_second_object": t.get("train_s_end_to_end_second_object"),
             "iters": t.get("iters"), "partial_d": t.get("partial_d"), "not_pruned_pct": t.get("not_pruned_pct"),
+            "pruned_vs_exact_agreement": t.get("pruned_vs_exact_agreement"),
             "stages": {nm: {"ms": s["ms"], "frac": s["frac"], "bound": s["bound"]} for nm, s in t.get("stages", {}).items()}}
 
 
@@ -579,7 +582,7 @@ def main():
             on, od, okk, oiters, ohier, ogen = CONFIGS[other]
             _capi.check(_capi.load().skm_device_cache_trim(0))
             others[other] = compact(run_config(args, other, on, od, okk, oiters, ohier, ogen, steps=2, warmup=1,
-                                               with_cpu=False, with_host=False, with_extras=False))
+                                               with_cpu=False, with_host=False, with_extras=False, with_agreement=True))
         out["other_configs"] = others
     print(json.dumps(out))
 

@@ -214,23 +214,27 @@ __global__ __launch_bounds__(PRUNE_WAVES * 64, 4) void prune_pool_kernel(PruneLi
                 const uint32_t incq = (uint32_t) __builtin_amdgcn_readlane((int) inc, q);
                 const uint2* list = a.cand + (int64_t) pq * a.cap;
                 const int cnt0 = cnt;
-                bool deferred = false;
+                bool deferred = false, keep_more = true;
                 uint2 e = ent[q];
                 for (;;) {
                     const bool mine = cur + (uint32_t) lane < nq && e.x / SKM_Y_BATCH_SIZE == (uint32_t) jb;
-                    const bool keep = mine && __uint_as_float(e.y) < thrq;
+                    const bool keep = keep_more && mine && __uint_as_float(e.y) < thrq;
                     const unsigned long long mask = __ballot(keep);
                     const int nk = __popcll(mask);
-                    if (cnt + nk > POOL_CAP) {  // the point waits for the next round (never the first of a round)
-                        deferred = true;
-                        break;
+                    if (cnt + nk > POOL_CAP) {
+                        // the point waits for the next round.  The first point of a round always fits (a batch holds
+                        // 1024 distinct centroids); a list that says otherwise is malformed, and its batch is cut short
+                        // rather than waited for forever
+                        deferred = cnt0 > 0;
+                        if (deferred) break;
+                        keep_more = false;
                     }
-                    if (keep) {
+                    if (keep && keep_more) {
                         const int slot = cnt + __popcll(mask & ((1ull << lane) - 1ull));
                         L.key[slot] = (uint16_t) ((q << POOL_Q_SHIFT) | (e.x - (uint32_t) base));
                         L.acc[slot] = __uint_as_float(e.y);
                     }
-                    cnt += nk;
+                    cnt += keep_more ? nk : 0;
                     const int run = __popcll(__ballot(mine));  // the entries of the batch are consecutive
                     cur += (uint32_t) run;
                     if (run < 64 || cur >= nq) break;

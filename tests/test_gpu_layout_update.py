@@ -234,3 +234,26 @@ def test_edit_rows_balancing_and_normalize(capi, ctx):
     nrm = np.linalg.norm(dC.download().astype(np.float64), axis=1)
     assert np.allclose(nrm, 1.0, atol=1e-5)  # test_superkmeans.cpp:376-407
     dC.free()
+
+
+def test_device_block_cache_limit_and_trim(capi, ctx):
+    """Released blocks are kept for reuse up to the cache's byte limit: with the limit at zero a freed block goes back
+    to the driver, with room it is handed out again by the next allocation of its size; trimming empties the cache.
+    Checked through the addresses the allocator returns (a block of an unusual size, so that nothing else takes it)."""
+    lib = ctx.lib
+    size = (37 << 20) + 512
+    capi.check(lib.skm_device_cache_trim(0))
+    try:
+        capi.check(lib.skm_device_cache_set_limit(0, 1 << 30))
+        a = ctx.empty(size // 4)
+        first = a.ptr
+        a.free()
+        b = ctx.empty(size // 4)
+        assert b.ptr == first  # came back from the cache
+        b.free()
+        capi.check(lib.skm_device_cache_set_limit(0, 0))  # the idle block leaves with the lowered limit
+        c = ctx.empty(size // 4)
+        c.free()  # nothing is kept now
+        capi.check(lib.skm_device_cache_trim(0))
+    finally:
+        capi.check(lib.skm_device_cache_set_limit(0, 48 << 30))

@@ -44,6 +44,12 @@ def _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=False, 
     return out
 
 
+def _last_overflow(capi, ctx):
+    over = ctypes.c_uint64()
+    capi.check(ctx.lib.skm_ctx_get_last_overflow(ctx.handle, ctypes.byref(over)))
+    return over.value
+
+
 def _setup(oracle, blobs, n, d, k, seed, std=0.3):
     X = blobs(n, d, k, std=std, seed=seed)
     g = np.random.default_rng(seed + 1)
@@ -193,7 +199,10 @@ def test_both_candidate_kernels_with_overflowing_lists(capi, ctx, oracle, blobs)
     ratios = np.minimum(1.0, 3.0 * oracle.ratios(d, 1.5)).astype(np.float32)  # looser still: most lists overflow
     ratios[d] = 1.0
     tiled = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=1)
+    over = _last_overflow(capi, ctx)
+    assert n // 2 < over <= n  # most points went through the second pass
     stationary = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=2)
+    assert _last_overflow(capi, ctx) == over
     big = _pruned(capi, ctx, oracle, X, C, prev, 40, ratios, kernel=3)
     assert np.array_equal(tiled[0], stationary[0]) and np.array_equal(tiled[0], big[0])
     assert np.array_equal(tiled[1].view(np.uint32), stationary[1].view(np.uint32))
@@ -288,6 +297,7 @@ def test_pruned_incumbent_only_survivor_keeps_seed_distance(capi, ctx, oracle):
     prev = np.array([0, 1, 0, 1], dtype=np.uint32)
     ratios = oracle.ratios(d, 1.5)
     gi, gd, gtotal, _ = _pruned(capi, ctx, oracle, X, C, prev, 32, ratios)
+    assert _last_overflow(capi, ctx) == 0
     assert np.array_equal(gi, prev)
     assert gtotal == 4
     full = ((X.astype(np.float64) - C[prev].astype(np.float64)) ** 2).sum(1)
