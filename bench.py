@@ -428,13 +428,12 @@ def assign_training_points_legs(_capi, km, Xhost, centroids, exact_assign, n, d,
         took = time.perf_counter() - t0
         prof = ctx.prof()
         ctx.prof_enable(False)
-        over = ctypes.c_uint64()
-        _capi.check(obj.lib.skm_ctx_get_last_overflow(ctx.handle, ctypes.byref(over)))
+        over = obj.training_overflow()
         ms = lambda nm: round(prof.get(nm, (0.0, 0))[0], 2)
         legs.append({"config": label, "ms_end_to_end_from_host_rows": round(took * 1e3, 1),
                      "points_per_s": round(n / took, 1),
                      "equals_exact_assign": round(float(np.mean(got == exact)), 6),
-                     "overflow_fraction": round(over.value / n, 4),
+                     "overflow_fraction": round(over / n, 4),
                      "device_ms": {"pruned_search": ms("search"), "seed": ms("search/seed"), "partial_gemm": ms("search/blas"),
                                    "list_walk": ms("search/pdx"), "second_pass": ms("search/overflow")}})
 

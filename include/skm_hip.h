@@ -102,6 +102,12 @@ int skm_download(skm_ctx* ctx, void* h_dst, const void* d_src, size_t bytes);
  * runtime stages it); pinned memory must stay unchanged until the context is synchronised (skm_sync,
  * skm_download or skm_upload). */
 int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
+/* Upload on the context's transfer stream that returns when the bytes are in device memory and leaves the context's
+ * own stream alone: meant for a second host thread that feeds slabs of rows while the first one queues the work on
+ * the slabs that have arrived (AssignTrainingPoints, reference superkmeans.h:397, takes host pointers only).  One
+ * transfer per context at a time (this call or skm_upload_overlapped); the first transfer of a context makes its
+ * transfer stream, so start no second one before that call has returned.  d_dst must not be in use by queued work. */
+int skm_upload_detached(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int skm_copy(skm_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
 int skm_fill_u32(skm_ctx* ctx, void* d_dst, uint32_t value, size_t count);
 
@@ -221,6 +227,11 @@ int skm_group_by_assignment(skm_ctx* ctx, const uint32_t* d_idx, size_t n, size_
  * out[index[j]] = local[j] + offset. */
 int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_t* d_local, size_t m,
                             uint32_t offset, uint32_t* d_out);
+/* The seeding of the unsampled points in AssignTrainingPoints (superkmeans.h:553-560): every entry of d_seeds that
+ * holds 0xffffffff becomes d_representative[d_group[i]] (the point's nearest meso-centroid, and one centroid of that
+ * meso-cluster); the other entries, the training assignments of the sampled points, stay. */
+int skm_seeds_from_groups(skm_ctx* ctx, uint32_t* d_seeds, const uint32_t* d_group, const uint32_t* d_representative,
+                          size_t n);
 /* BatchComputer::FindKNearestNeighbors (batch_computers.h:191-274): for every row of x the k rows of
  * y with the smallest -2 x.y + ||x||^2 + ||y||^2, ordered by (distance, index), y taken in batches of
  * 1024 rows: entries kept from earlier batches compete with their distance clamped at 0, the result

@@ -100,6 +100,9 @@ int skm_kmeans_assign_training_points(skm_kmeans* km, const float* h_vectors, co
  * can compare them).  count must equal that call's n_vectors; SKM_ERR_RUNTIME when there was no such call or it fell
  * back to Assign. */
 int skm_kmeans_get_training_seeds(skm_kmeans* km, uint32_t* h_out, size_t count);
+/* How many vectors of that call left more candidates than a candidate list holds and went through the second pass of
+ * the pruned search (no counterpart in the reference, whose search keeps no lists; 0 before the first call). */
+int skm_kmeans_get_training_overflow(skm_kmeans* km, uint64_t* out_points);
 
 /* Test hook, no counterpart in the reference: SplitClusters of the object's class (flat: superkmeans.h:890-928;
  * hierarchical: hierarchical_superkmeans.h:579-678) on a given state.  h_centroids (k x d) and h_sizes (k) are replaced

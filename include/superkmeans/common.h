@@ -5,11 +5,15 @@
 
 #include <algorithm>
 #include <cmath>
+#include <condition_variable>
 #include <cstddef>
 #include <cstdint>
+#include <exception>
+#include <mutex>
 #include <random>
 #include <stdexcept>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "skm_hip.h"
@@ -288,6 +292,64 @@ class Buffer {
     skm_ctx* ctx_ = nullptr;
     T* ptr_ = nullptr;
     size_t count_ = 0;
+};
+
+// Sends host rows to the device in slabs from a thread of its own (skm_upload_detached), so that the caller's thread
+// can queue the work on every slab as soon as it has arrived, whatever that work waits for in between.  WaitFor(i)
+// returns when slab i is in device memory and rethrows what the transfer thread failed with.
+class RowFeeder {
+  public:
+    RowFeeder(skm_ctx* ctx, float* d_dst, const float* h_src, size_t n_rows, size_t row_floats, size_t slab_rows)
+        : n_slabs_((n_rows + slab_rows - 1) / slab_rows) {
+        worker_ = std::thread([this, ctx, d_dst, h_src, n_rows, row_floats, slab_rows] {
+            try {
+                for (size_t s = 0; s < n_slabs_; ++s) {
+                    {
+                        std::lock_guard<std::mutex> lock(mutex_);
+                        if (stop_) return;
+                    }
+                    const size_t r0 = s * slab_rows, m = std::min(slab_rows, n_rows - r0);
+                    Check(skm_upload_detached(ctx, d_dst + r0 * row_floats, h_src + r0 * row_floats,
+                                              m * row_floats * sizeof(float)));
+                    {
+                        std::lock_guard<std::mutex> lock(mutex_);
+                        landed_ = s + 1;
+                    }
+                    arrived_.notify_all();
+                }
+            } catch (...) {
+                {
+                    std::lock_guard<std::mutex> lock(mutex_);
+                    error_ = std::current_exception();
+                }
+                arrived_.notify_all();
+            }
+        });
+    }
+    ~RowFeeder() {
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            stop_ = true;
+        }
+        if (worker_.joinable()) worker_.join();
+    }
+    RowFeeder(const RowFeeder&) = delete;
+    RowFeeder& operator=(const RowFeeder&) = delete;
+    size_t NumSlabs() const { return n_slabs_; }
+    void WaitFor(size_t slab) {
+        std::unique_lock<std::mutex> lock(mutex_);
+        arrived_.wait(lock, [&] { return landed_ > slab || error_; });
+        if (landed_ <= slab) std::rethrow_exception(error_);
+    }
+
+  private:
+    const size_t n_slabs_;
+    std::thread worker_;
+    std::mutex mutex_;
+    std::condition_variable arrived_;
+    size_t landed_ = 0;
+    bool stop_ = false;
+    std::exception_ptr error_;
 };
 
 } // namespace hip

@@ -236,24 +236,25 @@ class SuperKMeans {
         }
         partial_d = std::max<uint32_t>(MIN_PARTIAL_D, vertical_d / 2);
 
-        // The caller's vectors go to the device in slabs; every slab is rotated while the next one is copied
-        // (already rotated vectors are used as they arrive).  The raw copy is kept for the seeding below.
+        // The caller's vectors go to the device in slabs, from a thread of their own; below, every slab is rotated
+        // and searched while the later ones are still on their way (already rotated vectors are used as they arrive).
         dbuf<float> d_rot(ctx, n_vectors * d), d_raw;
         if (!config.data_already_rotated) d_raw.Reset(ctx, n_vectors * d);
         dbuf<float>& landing = config.data_already_rotated ? d_rot : d_raw;
-        {
-            const size_t slab = UploadSlabRows();
-            for (size_t r0 = 0; r0 < n_vectors; r0 += slab) {
-                const size_t m = std::min(slab, n_vectors - r0);
-                landing.UploadOverlapped(vectors + r0 * d, m * d, r0 * d);
-                if (!config.data_already_rotated) pruner->Rotate(ctx, d_raw.get() + r0 * d, d_rot.get() + r0 * d, m);
-            }
-        }
+        const size_t slab = UploadSlabRows();
+        hip::RowFeeder feed(ctx, landing.get(), vectors, n_vectors, d, slab);
         // Final centroids: horizontal_centroids / centroids (PDX) / partial_horizontal_centroids were
         // all refreshed by the last ConsolidateCentroids.
         hip::Check(skm_norms(ctx, horizontal_centroids.get(), n_centroids, d, partial_d, centroid_norms.get()));
+        EnsurePdxLayout(horizontal_centroids.get(), n_centroids);
 
+        // Seeds that do not depend on the vectors are made here; an entry of NO_SEED is resolved on the device, slab
+        // by slab, from the nearest meso-centroid of the vector.
+        constexpr uint32_t NO_SEED = 0xffffffffu;
         std::vector<uint32_t> seeds(n_vectors);
+        dbuf<float> d_meso;
+        dbuf<uint32_t> d_meso_to_original, d_meso_assignments;
+        size_t n_meso = 0;
         if (config.sampling_fraction == 1.0f) {
             std::memcpy(seeds.data(), assignments.get(), n_vectors * sizeof(uint32_t));
         } else if (config.sampling_fraction > 0.8f) {
@@ -277,49 +278,55 @@ class SuperKMeans {
             tmp_config.angular = config.angular;
             tmp_config.data_already_rotated = config.data_already_rotated;
             tmp_config.dct_rotation = config.dct_rotation;
-            auto new_n_centroids = static_cast<size_t>(std::sqrt(n_centroids));
+            n_meso = static_cast<size_t>(std::sqrt(n_centroids));
             // Same dimensionality and seed as this object: the rotation matrix and ratios would come out the same,
             // so the tables are shared instead of being factorised again on the host (the hierarchical variant
             // holds tables with another epsilon and builds fresh ones, as the reference does).
             std::unique_ptr<SuperKMeans> tmp_owner(
                 pruner->Epsilon0() == PRUNER_INITIAL_THRESHOLD
-                    ? new SuperKMeans(new_n_centroids, d, tmp_config, pruner)
-                    : new SuperKMeans(new_n_centroids, d, tmp_config));
+                    ? new SuperKMeans(n_meso, d, tmp_config, pruner)
+                    : new SuperKMeans(n_meso, d, tmp_config));
             SuperKMeans& tmp_kmeans = *tmp_owner;
             auto meso_centroids = tmp_kmeans.Train(centroids, n_centroids);
-            // Nearest meso-centroid of every vector, on the copy that is already on the device.
-            hip::Check(skm_sync(ctx));
-            std::vector<uint32_t> meso_assignments(n_vectors);
-            {
-                skm_ctx* tctx = tmp_kmeans.GetContext();
-                dbuf<float> d_meso(tctx, new_n_centroids * d);
-                d_meso.Upload(meso_centroids.data(), new_n_centroids * d);
-                dbuf<uint32_t> d_meso_assignments(tctx, n_vectors);
-                tmp_kmeans.AssignDevice(landing.get(), d_meso.get(), n_vectors, new_n_centroids, d_meso_assignments.get());
-                d_meso_assignments.Download(meso_assignments.data(), n_vectors);
-            }
-            auto centroids_to_meso = tmp_kmeans.Assign(centroids, meso_centroids.data(), n_centroids, new_n_centroids);
+            auto centroids_to_meso = tmp_kmeans.Assign(centroids, meso_centroids.data(), n_centroids, n_meso);
             g_n_threads = n_threads;
-            std::vector<uint32_t> meso_to_original(new_n_centroids, 0);
+            std::vector<uint32_t> meso_to_original(n_meso, 0);
             for (size_t c = 0; c < n_centroids; ++c) meso_to_original[centroids_to_meso[c]] = static_cast<uint32_t>(c);
-            size_t cur = 0;
-            for (; cur < n_samples; ++cur) seeds[sampled_indices[cur]] = assignments[cur];
-            for (; cur < n_vectors; ++cur) {
-                const size_t orig_idx = sampled_indices[cur];
-                seeds[orig_idx] = meso_to_original[meso_assignments[orig_idx]];
-            }
+            d_meso.Reset(ctx, n_meso * d);
+            d_meso.Upload(meso_centroids.data(), n_meso * d);
+            d_meso_to_original.Reset(ctx, n_meso);
+            d_meso_to_original.Upload(meso_to_original.data(), n_meso);
+            d_meso_assignments.Reset(ctx, n_vectors);
+            std::fill(seeds.begin(), seeds.end(), NO_SEED);
+            for (size_t cur = 0; cur < n_samples; ++cur) seeds[sampled_indices[cur]] = assignments[cur];
         }
-        dbuf<uint32_t> d_seed(ctx, n_vectors);
+        dbuf<uint32_t> d_seed(ctx, n_vectors), d_first_seed;
         d_seed.Upload(seeds.data(), n_vectors);
-        training_seeds = std::move(seeds);
+        if (n_meso > 0) d_first_seed.Reset(ctx, n_vectors);
         dbuf<float> d_norms_p(ctx, n_vectors), d_dist(ctx, n_vectors);
-        hip::Check(skm_norms(ctx, d_rot.get(), n_vectors, d, partial_d, d_norms_p.get()));
-        uint64_t not_pruned_total = 0;
-        EnsurePdxLayout(horizontal_centroids.get(), n_centroids);
-        hip::Check(skm_assign_pruned(ctx, d_rot.get(), n_vectors, horizontal_centroids.get(), this->centroids.get(),
-                                     partial_horizontal_centroids.get(), n_clusters, d, vertical_d, partial_d,
-                                     pruner->DeviceRatios(), d_norms_p.get(), centroid_norms.get(), d_seed.get(),
-                                     d_dist.get(), &not_pruned_total, nullptr));
+        training_overflow_points = 0;
+        for (size_t r0 = 0, s = 0; r0 < n_vectors; r0 += slab, ++s) {
+            const size_t m = std::min(slab, n_vectors - r0);
+            feed.WaitFor(s);
+            if (!config.data_already_rotated) pruner->Rotate(ctx, d_raw.get() + r0 * d, d_rot.get() + r0 * d, m);
+            if (n_meso > 0) {
+                // nearest meso-centroid in the space the caller's centroids are in, then the seeds still open
+                AssignDevice(landing.get() + r0 * d, d_meso.get(), m, n_meso, d_meso_assignments.get() + r0);
+                hip::Check(skm_seeds_from_groups(ctx, d_seed.get() + r0, d_meso_assignments.get() + r0,
+                                                 d_meso_to_original.get(), m));
+                hip::Check(skm_copy(ctx, d_first_seed.get() + r0, d_seed.get() + r0, m * sizeof(uint32_t)));
+            }
+            hip::Check(skm_norms(ctx, d_rot.get() + r0 * d, m, d, partial_d, d_norms_p.get() + r0));
+            hip::Check(skm_assign_pruned(ctx, d_rot.get() + r0 * d, m, horizontal_centroids.get(), this->centroids.get(),
+                                         partial_horizontal_centroids.get(), n_clusters, d, vertical_d, partial_d,
+                                         pruner->DeviceRatios(), d_norms_p.get() + r0, centroid_norms.get(),
+                                         d_seed.get() + r0, d_dist.get() + r0, nullptr, nullptr));
+            uint64_t overflowed = 0;
+            hip::Check(skm_ctx_get_last_overflow(ctx, &overflowed));
+            training_overflow_points += overflowed;
+        }
+        if (n_meso > 0) d_first_seed.Download(seeds.data(), n_vectors);
+        training_seeds = std::move(seeds);
         std::vector<uint32_t> result(n_vectors);
         d_seed.Download(result.data(), n_vectors);
         if (config.sampling_fraction == 1.0f) {
@@ -357,6 +364,9 @@ class SuperKMeans {
      *  builds them in place in its result array, superkmeans.h:454-563); empty before the first call and after a
      *  call that fell back to Assign. */
     [[nodiscard]] const std::vector<uint32_t>& GetTrainingSeeds() const noexcept { return training_seeds; }
+    /** How many vectors of the last pruned AssignTrainingPoints left more candidates than their list holds and took
+     *  the second pass of the search (no counterpart in the reference, whose search keeps no lists). */
+    [[nodiscard]] uint64_t GetTrainingOverflow() const noexcept { return training_overflow_points; }
     [[nodiscard]] float GetSamplingFraction() const noexcept { return config.sampling_fraction; }
     /** Host copy of the per-point squared distances of the last training iteration. */
     [[nodiscard]] distance_t* GetDistancesPointer() { return host_distances.data(); }
@@ -1076,6 +1086,7 @@ class SuperKMeans {
     dbuf<uint32_t> gt_assignments, promising_centroids;
     std::vector<float> host_distances;
     std::vector<uint32_t> training_seeds;  // GetTrainingSeeds
+    uint64_t training_overflow_points = 0;  // GetTrainingOverflow
     std::vector<centroid_value_t> prepared_centroids;  // PrepareHostOutputs
     std::thread host_outputs_thread;
     bool collect_prune_accounting = false;

@@ -36,6 +36,7 @@ _PROTOTYPES = {
     "skm_device_cache_set_limit": (c_int, [c_int, c_size_t]),
     "skm_upload": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_upload_overlapped": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "skm_upload_detached": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_householder_q": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "skm_download": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "skm_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t]),
@@ -68,6 +69,7 @@ _PROTOTYPES = {
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),
+    "skm_seeds_from_groups": (c_int, [c_void_p, _F, _F, _F, c_size_t]),
     "skm_knn": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_size_t, _F, _F, c_size_t, _F, _F]),
     "skm_recall_hits": (c_int, [c_void_p, _F, _F, _F, c_size_t, c_size_t, c_size_t, c_size_t, c_void_p]),
     "skm_synth_gaussian_mixture": (
@@ -92,6 +94,7 @@ _PROTOTYPES = {
     "skm_kmeans_get_stats": (c_int, [c_void_p, c_int, c_void_p, c_size_t]),
     "skm_kmeans_get_assignments": (c_int, [c_void_p, c_void_p, c_size_t]),
     "skm_kmeans_get_training_seeds": (c_int, [c_void_p, c_void_p, c_size_t]),
+    "skm_kmeans_get_training_overflow": (c_int, [c_void_p, POINTER(c_uint64)]),
     "skm_kmeans_split_clusters_on_state": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_size_t, POINTER(c_uint64)]),
     "skm_kmeans_context": (c_int, [c_void_p, POINTER(c_void_p)]),
     "skm_kmeans_set_prune_accounting": (c_int, [c_void_p, c_int]),
@@ -409,6 +412,11 @@ class KMeans:
         out = np.empty(count, dtype=np.uint32)
         check(self.lib.skm_kmeans_get_training_seeds(self.handle, out.ctypes.data, count))
         return out
+
+    def training_overflow(self):
+        out = c_uint64()
+        check(self.lib.skm_kmeans_get_training_overflow(self.handle, ctypes.byref(out)))
+        return int(out.value)
 
     @property
     def is_trained(self):

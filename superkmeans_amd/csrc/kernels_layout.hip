@@ -93,6 +93,14 @@ __global__ __launch_bounds__(256) void scatter_assignments_kernel(
     if (j < m) out[index[j]] = local[j] + offset;
 }
 
+__global__ __launch_bounds__(256) void seeds_from_groups_kernel(
+    uint32_t* __restrict__ seeds, const uint32_t* __restrict__ group, const uint32_t* __restrict__ representative,
+    size_t n
+) {
+    const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n && seeds[i] == 0xffffffffu) seeds[i] = representative[group[i]];
+}
+
 } // namespace skm
 
 using namespace skm;
@@ -141,6 +149,17 @@ int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_
     hipLaunchKernelGGL(scatter_assignments_kernel, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, ctx->stream, d_index,
                        d_local, m, offset, d_out);
     return check_hip(hipGetLastError(), "scatter_assignments_kernel launch");
+}
+
+int skm_seeds_from_groups(skm_ctx* ctx, uint32_t* d_seeds, const uint32_t* d_group, const uint32_t* d_representative,
+                          size_t n) {
+    SKM_REQUIRE(ctx, "null context");
+    if (n == 0) return SKM_OK;
+    SKM_REQUIRE(d_seeds && d_group && d_representative, "null pointer");
+    SKM_REQUIRE((n + 255) / 256 <= 0x7fffffffULL, "too many points");
+    hipLaunchKernelGGL(seeds_from_groups_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, ctx->stream, d_seeds,
+                       d_group, d_representative, n);
+    return check_hip(hipGetLastError(), "seeds_from_groups_kernel launch");
 }
 
 } // extern "C"

@@ -407,31 +407,49 @@ int skm_upload(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
     return SKM_OK;
 }
 
+namespace {
+// The transfer stream of a context and the events that order it before the context's stream, made on first use.
+int ensure_copy_stream(skm_ctx* ctx) {
+    if (ctx->copy_stream) return SKM_OK;
+    hipStream_t s = nullptr;
+    SKM_HIP_TRY(hipStreamCreate(&s));
+    for (auto& e : ctx->copy_done) {
+        const hipError_t rc = hipEventCreateWithFlags(&e, hipEventDisableTiming);
+        if (rc != hipSuccess) {
+            for (auto& made : ctx->copy_done) {
+                if (made) (void) hipEventDestroy(made);
+                made = nullptr;
+            }
+            (void) hipStreamDestroy(s);
+            return check_hip(rc, "hipEventCreateWithFlags");
+        }
+    }
+    ctx->copy_stream = s;
+    return SKM_OK;
+}
+} // namespace
+
 int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
     SKM_REQUIRE(ctx, "null context");
     if (bytes == 0) return SKM_OK;
     SKM_REQUIRE(d_dst && h_src, "null pointer");
     SKM_HIP_TRY(hipSetDevice(ctx->device));
-    if (!ctx->copy_stream) {
-        hipStream_t s = nullptr;
-        SKM_HIP_TRY(hipStreamCreate(&s));
-        for (auto& e : ctx->copy_done) {
-            const hipError_t rc = hipEventCreateWithFlags(&e, hipEventDisableTiming);
-            if (rc != hipSuccess) {
-                for (auto& made : ctx->copy_done) {
-                    if (made) (void) hipEventDestroy(made);
-                    made = nullptr;
-                }
-                (void) hipStreamDestroy(s);
-                return check_hip(rc, "hipEventCreateWithFlags");
-            }
-        }
-        ctx->copy_stream = s;
-    }
+    SKM_TRY(ensure_copy_stream(ctx));
     hipEvent_t done = ctx->copy_done[ctx->copy_seq++ % 8];
     SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->copy_stream));
     SKM_HIP_TRY(hipEventRecord(done, ctx->copy_stream));
     SKM_HIP_TRY(hipStreamWaitEvent(ctx->stream, done, 0));
+    return SKM_OK;
+}
+
+int skm_upload_detached(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
+    SKM_REQUIRE(ctx, "null context");
+    if (bytes == 0) return SKM_OK;
+    SKM_REQUIRE(d_dst && h_src, "null pointer");
+    SKM_HIP_TRY(hipSetDevice(ctx->device));
+    SKM_TRY(ensure_copy_stream(ctx));
+    SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->copy_stream));
+    SKM_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
     return SKM_OK;
 }
 

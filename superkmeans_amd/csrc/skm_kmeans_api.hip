@@ -259,6 +259,12 @@ int skm_kmeans_get_training_seeds(skm_kmeans* km, uint32_t* h_out, size_t count)
     return SKM_OK;
 }
 
+int skm_kmeans_get_training_overflow(skm_kmeans* km, uint64_t* out_points) {
+    if (!km || !out_points) return skm::set_error(SKM_ERR_INVALID, "null argument");
+    *out_points = km->base()->GetTrainingOverflow();
+    return SKM_OK;
+}
+
 int skm_kmeans_context(skm_kmeans* km, skm_ctx** out) {
     if (!km || !out) return skm::set_error(SKM_ERR_INVALID, "null argument");
     *out = km->base()->GetContext();

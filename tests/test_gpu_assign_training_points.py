@@ -15,6 +15,8 @@ where the point's two best centroids are within 1e-5 relative, at most 0.01 % of
 (a pruned one included, possibly after a split) the states agree to rounding only through a chaotic step, and the
 bar is the looser one described at _compare.
 """
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -111,3 +113,47 @@ def test_meso_centroid_seeding_on_data_that_is_already_rotated(capi, ctx, oracle
     bi, _, _ = oracle.brute_force(Xrot, OC)
     assert np.mean(got == bi) >= 0.995
     km.close()
+
+
+def test_vectors_that_arrive_in_several_slabs(capi, ctx, oracle, blobs):
+    """The vectors reach the device in slabs of 256 MiB (65,536 rows of 1024 dimensions) and every slab is seeded and
+    searched while the later ones are on their way.  Points are independent in the search, so the result must be the
+    one of a single pruned search over all points from the same seeds, bit for bit.  data_already_rotated, so that
+    the rows and centroids the object searches are the caller's own; few samples, so that most seeds are resolved
+    on the device from the nearest meso-centroid of the slab's rows."""
+    n, d, k = 150_000, 1024, 1300
+    X = blobs(n, d, k, std=0.3, seed=5)
+    cfg = dict(iters=2, sampling_fraction=0.3, early_termination=0, seed=42, suppress_warnings=1,
+               max_points_per_cluster=99999, data_already_rotated=1)
+    km = capi.KMeans(k, d, **cfg)
+    C = km.train(X)
+    got = km.assign_training_points(X, C)
+    seeds = km.training_seeds(n)
+    overflowed = km.training_overflow()
+    km.close()
+    assert seeds.max() < k and len(np.unique(seeds)) > 1
+    H, V = oracle.dimension_split(d)
+    partial_d = max(16, V // 2)
+    _, ratios = capi.pruner_tables(d, 1.5, 42, 0)
+    dX, dC = ctx.array(X), ctx.array(C)
+    dP, dA = ctx.empty(k * d), ctx.empty((k, V))
+    capi.check(ctx.lib.skm_pdxify(ctx.handle, dC.ptr, k, d, V, dP.ptr, dA.ptr))
+    xn, cn = ctx.empty(n), ctx.empty(k)
+    capi.check(ctx.lib.skm_norms(ctx.handle, dX.ptr, n, d, partial_d, xn.ptr))
+    capi.check(ctx.lib.skm_norms(ctx.handle, dC.ptr, k, d, partial_d, cn.ptr))
+    dR = ctx.array(ratios)
+    idx, dist = ctx.array(seeds), ctx.empty(n)
+    capi.check(ctx.lib.skm_assign_pruned(ctx.handle, dX.ptr, n, dC.ptr, dP.ptr, dA.ptr, k, d, V, partial_d, dR.ptr,
+                                         xn.ptr, cn.ptr, idx.ptr, dist.ptr, None, None))
+    whole = idx.download()
+    over = ctypes.c_uint64()
+    capi.check(ctx.lib.skm_ctx_get_last_overflow(ctx.handle, ctypes.byref(over)))
+    for a in (dX, dC, dP, dA, xn, cn, dR, idx, dist):
+        a.free()
+    assert np.array_equal(got, whole), f"{np.sum(got != whole)} of {n} points differ"
+    assert overflowed == over.value
+    # the seeds of the unsampled points are representatives of meso-clusters: about sqrt(k) distinct values among them
+    values, counts = np.unique(seeds, return_counts=True)
+    assert np.sum(counts >= 0.2 * n / np.sqrt(k)) <= int(np.sqrt(k))
+    bi, _, _ = oracle.brute_force(X[:4096], C)
+    assert np.mean(got[:4096] == bi) >= 0.995

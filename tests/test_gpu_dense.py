@@ -217,6 +217,46 @@ def test_upload_on_the_transfer_stream_orders_before_later_work(capi, ctx):
     dX.free(), out.free()
 
 
+def test_detached_upload_from_a_second_thread(capi, ctx):
+    """skm_upload_detached returns when the bytes are in device memory and leaves the context's stream alone: a second
+    thread feeds the slabs while this one queues the norms of every slab that has arrived."""
+    import threading
+
+    g = np.random.default_rng(8)
+    n, d, slab = 50000, 512, 6000
+    X = g.standard_normal((n, d)).astype(np.float32)
+    dX, out = ctx.empty((n, d)), ctx.empty(n)
+    starts = list(range(0, n, slab))
+    arrived = [threading.Event() for _ in starts]
+    failed = []
+
+    def feed():
+        try:
+            for s, r0 in enumerate(starts):
+                m = min(slab, n - r0)
+                capi.check(ctx.lib.skm_upload_detached(ctx.handle, dX.ptr + r0 * d * 4, X[r0:r0 + m].ctypes.data, m * d * 4))
+                arrived[s].set()
+        except Exception as e:  # reported below, in the thread that runs the test
+            failed.append(e)
+            for a in arrived:
+                a.set()
+
+    t = threading.Thread(target=feed)
+    t.start()
+    for s, r0 in enumerate(starts):
+        assert arrived[s].wait(60)
+        assert not failed, failed
+        m = min(slab, n - r0)
+        capi.check(ctx.lib.skm_norms(ctx.handle, dX.ptr + r0 * d * 4, m, d, d, out.ptr + r0 * 4))
+    t.join()
+    ctx.sync()
+    assert np.array_equal(dX.download(), X)
+    assert np.allclose(out.download(), (X.astype(np.float64) ** 2).sum(1), rtol=1e-5)
+    capi.check(ctx.lib.skm_upload_detached(ctx.handle, dX.ptr, X.ctypes.data, 0))
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_upload_detached(ctx.handle, None, X.ctypes.data, 16))
+    dX.free(), out.free()
+
 
 def test_large_download_through_the_lanes_is_byte_exact(capi, ctx):
     """From 64 MiB a download goes through four threads, each moving every fourth 4 MiB chunk through its own pinned

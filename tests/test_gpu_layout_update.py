@@ -257,3 +257,20 @@ def test_device_block_cache_limit_and_trim(capi, ctx):
         capi.check(lib.skm_device_cache_trim(0))
     finally:
         capi.check(lib.skm_device_cache_set_limit(0, 48 << 30))
+
+
+def test_seeds_from_groups(capi, ctx):
+    """skm_seeds_from_groups: open entries (0xffffffff) take the representative of the point's group, the others stay."""
+    g = np.random.default_rng(3)
+    n, groups = 100_003, 37
+    seeds = g.integers(0, 5000, n, dtype=np.uint32)
+    seeds[g.random(n) < 0.7] = 0xFFFFFFFF
+    group = g.integers(0, groups, n, dtype=np.uint32)
+    rep = g.integers(0, 5000, groups, dtype=np.uint32)
+    dS, dG, dR = ctx.array(seeds), ctx.array(group), ctx.array(rep)
+    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, n))
+    want = np.where(seeds == 0xFFFFFFFF, rep[group], seeds)
+    assert np.array_equal(dS.download(), want)
+    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, 0))
+    for a in (dS, dG, dR):
+        a.free()
