@@ -131,9 +131,9 @@ def _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, cfg, gs, os_):
     deterministic, so they are repeated with 1, 2, ... iterations (centroids left in the rotated space) up to the
     iteration in question:
       * the first iteration in which any assignment differs follows a state that is the same on both sides, and
-        every point it assigns differently has its two candidates at almost the same distance (relative gap <= 2e-3
-        against the oracle's centroids: a split twin differs from its donor by 1 +/- 1/1024 per column); such points
-        are few (<= 0.1 %);
+        every point it assigns differently chose between a split twin and its donor (rows that differ by the
+        factors 1 +/- 1/1024 per column, relative gap <= 2e-3 against the oracle's centroids) or between two
+        centroids at the same distance to rounding (relative gap <= 1e-4); such points are few (<= 0.1 %);
       * from its own state of the iteration before, the device does what the oracle does: the oracle's pruned search
         started from the device's centroids and assignments returns the device's next assignments."""
     first = next((i for i, (a, b) in enumerate(zip(gs, os_))
@@ -162,7 +162,13 @@ def _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, cfg, gs, os_):
     dg = ((x64 - c64[ga[mism]]) ** 2).sum(1)
     do = ((x64 - c64[oa[mism]]) ** 2).sum(1)
     gap = np.abs(dg - do) / np.maximum(np.minimum(dg, do), 1e-12)
-    assert np.all(gap <= 2e-3), f"iteration {parted}: a differing point is no near tie (largest gap {gap.max():.2e})"
+    # the two candidates are a split twin and its donor (rows equal up to the factors 1 +/- 1/1024), or a tie to the
+    # rounding of the distances (which are differences of norms some ten times their size)
+    twins = np.max(np.abs(c64[ga[mism]] - c64[oa[mism]]), axis=1) <= (2.5 / 1024) * np.max(np.abs(c64[oa[mism]]), axis=1)
+    assert np.all(twins | (gap <= 1e-4)), (
+        f"iteration {parted}: a differing point is neither a near tie nor between twins "
+        f"(largest gap outside twins {gap[~twins].max():.2e})")
+    assert np.all(gap <= 2e-3), f"iteration {parted}: largest gap {gap.max():.2e}"
     ga_prev, gc_prev = states[first][0], states[first][1]
     ga_next, st = states[first + 1][0], states[first + 1][4]
     assert not st.is_gemm_only
