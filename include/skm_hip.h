@@ -105,8 +105,9 @@ int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t b
 /* Upload on the context's transfer stream that returns when the bytes are in device memory and leaves the context's
  * own stream alone: meant for a second host thread that feeds slabs of rows while the first one queues the work on
  * the slabs that have arrived (AssignTrainingPoints, reference superkmeans.h:397, takes host pointers only).  One
- * transfer per context at a time (this call or skm_upload_overlapped); the first transfer of a context makes its
- * transfer stream, so start no second one before that call has returned.  d_dst must not be in use by queued work. */
+ * transfer per context at a time (this call or skm_upload_overlapped).  The first call on a context makes its transfer
+ * stream: make that call (zero bytes will do) on the thread that owns the context before a feeder thread starts.
+ * d_dst must not be in use by queued work. */
 int skm_upload_detached(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes);
 int skm_copy(skm_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
 int skm_fill_u32(skm_ctx* ctx, void* d_dst, uint32_t value, size_t count);

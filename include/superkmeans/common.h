@@ -295,20 +295,22 @@ class Buffer {
 };
 
 // Sends host rows to the device in slabs from a thread of its own (skm_upload_detached), so that the caller's thread
-// can queue the work on every slab as soon as it has arrived, whatever that work waits for in between.  WaitFor(i)
-// returns when slab i is in device memory and rethrows what the transfer thread failed with.
+// can queue the work on every slab as soon as it has arrived, whatever that work waits for in between.  Slab s holds
+// the rows [edges[s], edges[s + 1]).  WaitFor(s) returns when slab s is in device memory and rethrows what the
+// transfer thread failed with.
 class RowFeeder {
   public:
-    RowFeeder(skm_ctx* ctx, float* d_dst, const float* h_src, size_t n_rows, size_t row_floats, size_t slab_rows)
-        : n_slabs_((n_rows + slab_rows - 1) / slab_rows) {
-        worker_ = std::thread([this, ctx, d_dst, h_src, n_rows, row_floats, slab_rows] {
+    RowFeeder(skm_ctx* ctx, float* d_dst, const float* h_src, size_t row_floats, std::vector<size_t> edges)
+        : edges_(std::move(edges)) {
+        Check(skm_upload_detached(ctx, d_dst, h_src, 0));  // the context's transfer stream exists before the thread does
+        worker_ = std::thread([this, ctx, d_dst, h_src, row_floats] {
             try {
-                for (size_t s = 0; s < n_slabs_; ++s) {
+                for (size_t s = 0; s + 1 < edges_.size(); ++s) {
                     {
                         std::lock_guard<std::mutex> lock(mutex_);
                         if (stop_) return;
                     }
-                    const size_t r0 = s * slab_rows, m = std::min(slab_rows, n_rows - r0);
+                    const size_t r0 = edges_[s], m = edges_[s + 1] - r0;
                     Check(skm_upload_detached(ctx, d_dst + r0 * row_floats, h_src + r0 * row_floats,
                                               m * row_floats * sizeof(float)));
                     {
@@ -335,7 +337,9 @@ class RowFeeder {
     }
     RowFeeder(const RowFeeder&) = delete;
     RowFeeder& operator=(const RowFeeder&) = delete;
-    size_t NumSlabs() const { return n_slabs_; }
+    size_t NumSlabs() const { return edges_.size() - 1; }
+    size_t FirstRow(size_t slab) const { return edges_[slab]; }
+    size_t Rows(size_t slab) const { return edges_[slab + 1] - edges_[slab]; }
     void WaitFor(size_t slab) {
         std::unique_lock<std::mutex> lock(mutex_);
         arrived_.wait(lock, [&] { return landed_ > slab || error_; });
@@ -343,7 +347,7 @@ class RowFeeder {
     }
 
   private:
-    const size_t n_slabs_;
+    const std::vector<size_t> edges_;  // ascending row offsets, the first 0, the last the number of rows
     std::thread worker_;
     std::mutex mutex_;
     std::condition_variable arrived_;

@@ -196,6 +196,17 @@ class SuperKMeans {
         return result;
     }
 
+    // Row offsets, from 0 to n_rows, of the slabs that AssignTrainingPoints searches one by one: UploadSlabRows() rows,
+    // but at least 65,536 (the kernels of the pruned search that are made for many points need 49,152 of them).
+    // Measured on 1 M rows of 1024 dimensions (reference defaults): slabs of 64 MiB (16,384 rows) 420 ms, 256 MiB 229 ms,
+    // 512 MiB 225 ms but 320 ms for the first call (the scratch memory of a slab's search grows with it); a smaller
+    // first slab changed nothing.
+    std::vector<size_t> UploadSlabEdges(const size_t n_rows) const {
+        std::vector<size_t> edges{0};
+        const size_t rows = std::max<size_t>(UploadSlabRows(), 65536);
+        while (edges.back() < n_rows) edges.push_back(std::min(n_rows, edges.back() + rows));
+        return edges;
+    }
     // Rows per slab of a host-to-device transfer that overlaps with compute: 256 MiB of rows, a multiple of 256.
     size_t UploadSlabRows() const {
         const size_t rows = (size_t(256) << 20) / (d * sizeof(float));
@@ -241,8 +252,7 @@ class SuperKMeans {
         dbuf<float> d_rot(ctx, n_vectors * d), d_raw;
         if (!config.data_already_rotated) d_raw.Reset(ctx, n_vectors * d);
         dbuf<float>& landing = config.data_already_rotated ? d_rot : d_raw;
-        const size_t slab = UploadSlabRows();
-        hip::RowFeeder feed(ctx, landing.get(), vectors, n_vectors, d, slab);
+        hip::RowFeeder feed(ctx, landing.get(), vectors, d, UploadSlabEdges(n_vectors));
         // Final centroids: horizontal_centroids / centroids (PDX) / partial_horizontal_centroids were
         // all refreshed by the last ConsolidateCentroids.
         hip::Check(skm_norms(ctx, horizontal_centroids.get(), n_centroids, d, partial_d, centroid_norms.get()));
@@ -305,8 +315,8 @@ class SuperKMeans {
         if (n_meso > 0) d_first_seed.Reset(ctx, n_vectors);
         dbuf<float> d_norms_p(ctx, n_vectors), d_dist(ctx, n_vectors);
         training_overflow_points = 0;
-        for (size_t r0 = 0, s = 0; r0 < n_vectors; r0 += slab, ++s) {
-            const size_t m = std::min(slab, n_vectors - r0);
+        for (size_t s = 0; s < feed.NumSlabs(); ++s) {
+            const size_t r0 = feed.FirstRow(s), m = feed.Rows(s);
             feed.WaitFor(s);
             if (!config.data_already_rotated) pruner->Rotate(ctx, d_raw.get() + r0 * d, d_rot.get() + r0 * d, m);
             if (n_meso > 0) {

@@ -444,10 +444,10 @@ int skm_upload_overlapped(skm_ctx* ctx, void* d_dst, const void* h_src, size_t b
 
 int skm_upload_detached(skm_ctx* ctx, void* d_dst, const void* h_src, size_t bytes) {
     SKM_REQUIRE(ctx, "null context");
+    SKM_HIP_TRY(hipSetDevice(ctx->device));
+    SKM_TRY(ensure_copy_stream(ctx));  // also for zero bytes: the owner's way to make the stream before a feeder starts
     if (bytes == 0) return SKM_OK;
     SKM_REQUIRE(d_dst && h_src, "null pointer");
-    SKM_HIP_TRY(hipSetDevice(ctx->device));
-    SKM_TRY(ensure_copy_stream(ctx));
     SKM_HIP_TRY(hipMemcpyAsync(d_dst, h_src, bytes, hipMemcpyHostToDevice, ctx->copy_stream));
     SKM_HIP_TRY(hipStreamSynchronize(ctx->copy_stream));
     return SKM_OK;
