@@ -118,6 +118,12 @@ int workspace(skm_ctx* ctx, int slot, size_t bytes, void** out) {
     if (slot < 0 || slot >= skm_ctx::WS_SLOTS) return set_error(SKM_ERR_INVALID, "bad workspace slot");
     if (ctx->ws_bytes[slot] < bytes) {
         if (ctx->ws[slot]) {
+            // a slot that grows again gets a quarter more than it held: requests that creep up call after call (the
+            // dense rows of the overflowing points of one slab after another) would otherwise reallocate every time
+            // (within the workspace limit, unless the request itself is beyond it)
+            size_t roomy = ctx->ws_bytes[slot] + ctx->ws_bytes[slot] / 4;
+            if (roomy > ctx->workspace_limit) roomy = ctx->workspace_limit;
+            if (bytes < roomy) bytes = roomy;
             SKM_HIP_TRY(hipStreamSynchronize(ctx->stream));
             SKM_TRY(device_release(ctx->device, ctx->ws[slot]));
             ctx->ws[slot] = nullptr;
