@@ -155,17 +155,26 @@ def stage_table(n, d, k, ks, hierarchical, stats, acct, prof, V):
         add_stage("pdx_relayout", "hbm", calls("consolidate/pdxify") * (2.0 * 4 * k * d + 4.0 * k * V), ms("consolidate/pdxify"), PEAK_HBM_GBPS)
     if "prune" in stage:
         p = stage["prune"]
-        # `frac` divides algorithmic bytes by time: most of them are 256-byte gathers of centroid blocks that the caches
-        # serve, so it is a rate of useful bytes, not HBM traffic.  `measured_*`: the bytes that leave the L2s, from the
-        # counters; `ns_per_pair_block`: the unit that tracks the walk's progress.
-        p["frac_is"] = "algorithmic bytes / time / HBM peak (block gathers are mostly cache hits); measured_frac is counter bytes"
+        # Two rates.  Algorithmic bytes / time counts every 256-byte gather of a centroid block, most of which the
+        # caches serve: a rate of useful bytes that can exceed the HBM peak.  Counter bytes / time is what leaves the
+        # L2s: that one is `frac` whenever the counters of these kernel sources are on record (otherwise `frac` stays
+        # the algorithmic rate and `frac_is` says so).  `ns_per_pair_block` is the unit that tracks the walk's progress.
+        p["algorithmic_bytes"] = prune_bytes
+        p["algorithmic_achieved"] = p["achieved"]
+        p["algorithmic_frac"] = p["frac"]
         if blocks_visited > 0:
             p["pair_blocks_visited"] = blocks_visited
             p["ns_per_pair_block"] = round(p["ms"] * 1e6 / blocks_visited, 4)
         value, source = measured(MEASURED_PRUNE_TRAFFIC_BYTES, (n, d, k, len(stats)))
         p["measured_bytes"] = value
-        p["measured_frac"] = round(value / (p["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4) if value else None
         p["measured_from"] = source
+        if value:
+            p["achieved"] = round(value / (p["ms"] * 1e-3) / 1e9, 2)
+            p["frac"] = round(p["achieved"] / PEAK_HBM_GBPS, 4)
+            p["frac_is"] = "counter bytes (FETCH_SIZE, WRITE_SIZE of every launch of the stage) / time / HBM peak"
+        else:
+            p["frac_is"] = "algorithmic bytes / time / HBM peak (block gathers are mostly cache hits): no counter figure for this shape and these sources"
+        p["measured_frac"] = p["frac"] if value else None
     return stage
 
 
@@ -501,7 +510,9 @@ def compact(result):
             "train_s_end_to_end_second_object": t.get("train_s_end_to_end_second_object"),
             "iters": t.get("iters"), "partial_d": t.get("partial_d"), "not_pruned_pct": t.get("not_pruned_pct"),
             "pruned_vs_exact_agreement": t.get("pruned_vs_exact_agreement"),
-            "stages": {nm: {"ms": s["ms"], "frac": s["frac"], "bound": s["bound"]} for nm, s in t.get("stages", {}).items()}}
+            "stages": {nm: dict({"ms": s["ms"], "frac": s["frac"], "bound": s["bound"]},
+                                **({"frac_is": s["frac_is"]} if "frac_is" in s else {}))
+                       for nm, s in t.get("stages", {}).items()}}
 
 
 def main():
