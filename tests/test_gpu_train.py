@@ -126,8 +126,9 @@ def test_every_iteration_in_lockstep_with_oracle(capi, ctx, oracle, blobs, n, d,
         prev_state = (c_t, a_t)
 
 
-def _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, cfg, gs, os_):
-    """Where the two runs part by more than 1e-4 in WCSS, the parting must be explained by near ties.  Both runs are
+def _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, cfg, gs, os_, first=None):
+    """Where the two runs part by more than 1e-4 in WCSS (or from the iteration with index `first`, when the caller has
+    found the parting by a finer measure), the parting must be explained by near ties.  Both runs are
     deterministic, so they are repeated with 1, 2, ... iterations (centroids left in the rotated space) up to the
     iteration in question:
       * the first iteration in which any assignment differs follows a state that is the same on both sides, and
@@ -136,8 +137,9 @@ def _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, cfg, gs, os_):
         centroids at the same distance to rounding (relative gap <= 1e-4); such points are few (<= 0.1 %);
       * from its own state of the iteration before, the device does what the oracle does: the oracle's pruned search
         started from the device's centroids and assignments returns the device's next assignments."""
-    first = next((i for i, (a, b) in enumerate(zip(gs, os_))
-                  if abs(a.objective - b.objective_f64) > 1e-4 * b.objective_f64), None)
+    if first is None:
+        first = next((i for i, (a, b) in enumerate(zip(gs, os_))
+                      if abs(a.objective - b.objective_f64) > 1e-4 * b.objective_f64), None)
     if first is None or first == 0:
         assert first is None, "the exact first iteration already differs"
         return
@@ -228,6 +230,45 @@ def test_flat_train_matches_oracle(capi, ctx, oracle, blobs, n, d, k, iters):
     # AssignTrainingPoints >= 98 % agreement with Assign (test_assign.cpp:118-155)
     atp = km.assign_training_points(X, C)
     assert np.mean(atp == a1) >= 0.98
+    km.close()
+
+
+# Whole runs at the strict bar.  Two fp32 implementations part only where a point sits between two centroids at the
+# same distance to rounding, which in practice means between a split twin and its donor; of 76 randomly drawn
+# configurations about half had no such point that the two sides resolved differently, and those stayed together to
+# rounding.  So: every iteration's objective and shift within 1e-4 (measured: 1e-7) and the same control flow up to the
+# first iteration where that fails; if none fails, final centroids within 1e-4 relative L2 (measured: 6e-7) and at
+# most 0.01 % of the assignments different; if one does, the parting is examined point by point (twins or ties, and
+# the device's own next step is the oracle's step from the device's state) and the rest of the run keeps the loose
+# bars.  In the environment the suite was written in, the first six runs stay together and the last two part.
+@pytest.mark.parametrize("n,d,k,iters,early,angular,std", [
+    (5900, 768, 280, 4, 0, 0, 0.5), (16700, 128, 260, 5, 0, 1, 0.3), (11600, 256, 785, 4, 0, 0, 0.3),
+    (14607, 384, 282, 8, 1, 0, 0.1), (33384, 128, 566, 8, 0, 0, 0.2), (19226, 768, 462, 5, 1, 0, 0.3),
+    (30524, 128, 436, 5, 0, 0, 0.2), (16710, 512, 325, 7, 0, 0, 0.3)])
+def test_flat_train_at_the_strict_bar_until_a_tie_parts_the_runs(capi, ctx, oracle, blobs, n, d, k, iters, early, angular,
+                                                                 std):
+    X = blobs(n, d, k, std=std, seed=n + d)
+    cfg = dict(iters=iters, sampling_fraction=1.0, early_termination=early, seed=42, angular=angular, suppress_warnings=1)
+    km, ok = capi.KMeans(k, d, **cfg), oracle.KMeans(k, d, **cfg)
+    C, OC = km.train(X), ok.train(X)
+    gs, os_ = km.stats(), ok.stats()
+    together = lambda a, b: (abs(a.objective - b.objective_f64) <= 1e-4 * b.objective_f64 and
+                             abs(a.shift - b.shift) <= 1e-4 * b.shift + 1e-9)
+    first = next((i for i, (a, b) in enumerate(zip(gs, os_)) if not together(a, b)), None)
+    for a, b in list(zip(gs, os_))[:first]:
+        assert a.is_gemm_only == b.is_gemm_only and a.partial_d == b.partial_d and a.split == b.split
+        if not a.is_gemm_only:
+            assert abs(a.not_pruned_pct - b.not_pruned_pct) <= 2e-3 * b.not_pruned_pct + 1e-6
+    _, oa, _, _ = ok.state()
+    if first is None:
+        assert len(gs) == len(os_)
+        assert _rel_l2(C, OC) <= 1e-4
+        assert np.mean(km.assignments(n) != oa) <= 1e-4
+    else:
+        assert first >= 2, "the runs part before any split twin exists"
+        _first_divergence_is_made_of_near_ties(capi, oracle, X, k, d, dict(cfg, early_termination=0), gs, os_, first=first)
+        m = min(len(gs), len(os_))
+        assert abs(gs[m - 1].objective - os_[m - 1].objective_f64) <= 2e-3 * os_[m - 1].objective_f64
     km.close()
 
 
