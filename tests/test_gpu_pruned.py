@@ -302,3 +302,44 @@ def test_pruned_incumbent_only_survivor_keeps_seed_distance(capi, ctx, oracle):
     assert gtotal == 4
     full = ((X.astype(np.float64) - C[prev].astype(np.float64)) ** 2).sum(1)
     assert np.allclose(gd, full, rtol=1e-5)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_shapes_every_kernel_and_walk_same_bits(capi, ctx, oracle, blobs, seed):
+    """Ten seeded random shapes per case (1 to 5,000 points, 65 to 3,300 centroids, d from 128 to 1539 with and without
+    16-byte aligned rows, d' from 8 up to 400, tight and random seeds, the reference's ratios or looser ones): every
+    choice of candidate kernel, walk and number of walk launches returns the bits of the tiled kernel with the
+    one-point walk, and what differs from the oracle is a tie or the exact answer."""
+    g = np.random.default_rng(seed)
+    for case in range(10):
+        d = int(g.choice([128, 132, 192, 256, 260, 384, 512, 600, 768, 1024, 1280, 1536]))
+        if g.random() < 0.15:
+            d += int(g.integers(1, 4))
+        _, V = oracle.dimension_split(d)
+        k = int(g.integers(65, 3300))
+        n = int(g.integers(1, 5000))
+        partial_d = int(g.integers(8, max(9, min(V - 1, 400))))
+        random_seeds, accounting = bool(g.random() < 0.4), bool(g.random() < 0.5)
+        X, C, prev = _setup(oracle, blobs, max(n, k + 10), d, k, seed=1000 * seed + case)
+        X, prev = X[:n], prev[:n]
+        if random_seeds:
+            prev = g.integers(0, k, n).astype(np.uint32)
+        ratios = oracle.ratios(d, 1.5)
+        if g.random() < 0.2:
+            ratios = np.minimum(1.0, 2.5 * ratios).astype(np.float32)
+            ratios[d] = 1.0
+        what = f"n={n} d={d} k={k} d'={partial_d} random_seeds={random_seeds} accounting={accounting}"
+        base = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, kernel=1, walk=1)
+        for kernel, walk, launches in ((0, 0, 1), (2, 2, 1), (3, 3, 1), (1, 3, 3), (3, 2, 1000), (2, 1, 1)):
+            other = _pruned(capi, ctx, oracle, X, C, prev, partial_d, ratios, accounting=accounting, kernel=kernel,
+                            walk=walk, launches=launches)
+            try:
+                _same_bits(base, other)
+            except AssertionError as e:
+                raise AssertionError(f"{what}: kernel {kernel}, walk {walk}, {launches} launches") from e
+        oi, _, _ = oracle.find_nn_pruned(X, C, prev, partial_d, ratios)
+        bi, bbest, bsecond = oracle.brute_force(X, C)
+        mism = np.nonzero(base[0] != oi)[0]
+        tie = (bsecond - bbest) <= 1e-5 * np.maximum(bbest, 1e-12)
+        assert all(base[0][i] == bi[i] or tie[i] for i in mism), what
+        assert len(mism) <= max(1, int(1e-4 * n)), what
