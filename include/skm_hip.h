@@ -172,7 +172,8 @@ int skm_assign_full_noalloc(skm_ctx* ctx, const float* d_x, size_t n, const floa
  *   d_pdx      the same centroids in PDX layout, d_aux their first vertical_d columns
  *   d_ratios   d + 1 floats, ADSamplingPruner::ratios (pdx/adsampling.h:93-99)
  *   d_xnorm_p / d_cnorm_p  squared norms over the first partial_d columns
- *   d_inout_idx in: previous assignment (seed); out: new assignment
+ *   d_inout_idx in: previous assignment (seed; every entry below k, the search reads that centroid's row); out:
+ *               new assignment
  *   d_out_dist  out: squared distance to the new assignment (unclamped, as the reference)
  *   h_out_not_pruned  sum over points of the per-point not-pruned counts (input of TunePartialD,
  *                     superkmeans.h:1230-1241); synchronises.
@@ -230,9 +231,10 @@ int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_
                             uint32_t offset, uint32_t* d_out);
 /* The seeding of the unsampled points in AssignTrainingPoints (superkmeans.h:553-560): every entry of d_seeds that
  * holds 0xffffffff becomes d_representative[d_group[i]] (the point's nearest meso-centroid, and one centroid of that
- * meso-cluster); the other entries, the training assignments of the sampled points, stay. */
+ * meso-cluster; d_representative has n_groups entries and a group at or past n_groups counts as the last one); the
+ * other entries, the training assignments of the sampled points, stay. */
 int skm_seeds_from_groups(skm_ctx* ctx, uint32_t* d_seeds, const uint32_t* d_group, const uint32_t* d_representative,
-                          size_t n);
+                          size_t n_groups, size_t n);
 /* BatchComputer::FindKNearestNeighbors (batch_computers.h:191-274): for every row of x the k rows of
  * y with the smallest -2 x.y + ||x||^2 + ||y||^2, ordered by (distance, index), y taken in batches of
  * 1024 rows: entries kept from earlier batches compete with their distance clamped at 0, the result

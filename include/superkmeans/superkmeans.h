@@ -323,7 +323,7 @@ class SuperKMeans {
                 // nearest meso-centroid in the space the caller's centroids are in, then the seeds still open
                 AssignDevice(landing.get() + r0 * d, d_meso.get(), m, n_meso, d_meso_assignments.get() + r0);
                 hip::Check(skm_seeds_from_groups(ctx, d_seed.get() + r0, d_meso_assignments.get() + r0,
-                                                 d_meso_to_original.get(), m));
+                                                 d_meso_to_original.get(), n_meso, m));
                 hip::Check(skm_copy(ctx, d_first_seed.get() + r0, d_seed.get() + r0, m * sizeof(uint32_t)));
             }
             hip::Check(skm_norms(ctx, d_rot.get() + r0 * d, m, d, partial_d, d_norms_p.get() + r0));

@@ -69,7 +69,7 @@ _PROTOTYPES = {
     "skm_shift": (c_int, [c_void_p, _F, _F, c_size_t, c_size_t, POINTER(c_double)]),
     "skm_gather_rows": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, _F, _F, _F]),
     "skm_scatter_assignments": (c_int, [c_void_p, _F, _F, c_size_t, c_uint32, _F]),
-    "skm_seeds_from_groups": (c_int, [c_void_p, _F, _F, _F, c_size_t]),
+    "skm_seeds_from_groups": (c_int, [c_void_p, _F, _F, _F, c_size_t, c_size_t]),
     "skm_knn": (c_int, [c_void_p, _F, c_size_t, _F, c_size_t, c_size_t, _F, _F, c_size_t, _F, _F]),
     "skm_recall_hits": (c_int, [c_void_p, _F, _F, _F, c_size_t, c_size_t, c_size_t, c_size_t, c_void_p]),
     "skm_synth_gaussian_mixture": (

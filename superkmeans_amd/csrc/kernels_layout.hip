@@ -95,10 +95,13 @@ __global__ __launch_bounds__(256) void scatter_assignments_kernel(
 
 __global__ __launch_bounds__(256) void seeds_from_groups_kernel(
     uint32_t* __restrict__ seeds, const uint32_t* __restrict__ group, const uint32_t* __restrict__ representative,
-    size_t n
+    uint32_t n_groups, size_t n
 ) {
     const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n && seeds[i] == 0xffffffffu) seeds[i] = representative[group[i]];
+    if (i < n && seeds[i] == 0xffffffffu) {
+        const uint32_t g = group[i];
+        seeds[i] = representative[g < n_groups ? g : n_groups - 1];  // a group out of range reads no stray memory
+    }
 }
 
 } // namespace skm
@@ -152,13 +155,14 @@ int skm_scatter_assignments(skm_ctx* ctx, const uint64_t* d_index, const uint32_
 }
 
 int skm_seeds_from_groups(skm_ctx* ctx, uint32_t* d_seeds, const uint32_t* d_group, const uint32_t* d_representative,
-                          size_t n) {
+                          size_t n_groups, size_t n) {
     SKM_REQUIRE(ctx, "null context");
     if (n == 0) return SKM_OK;
     SKM_REQUIRE(d_seeds && d_group && d_representative, "null pointer");
+    SKM_REQUIRE(n_groups > 0 && n_groups <= 0xffffffffULL, "the number of groups must be in [1, 2^32)");
     SKM_REQUIRE((n + 255) / 256 <= 0x7fffffffULL, "too many points");
     hipLaunchKernelGGL(seeds_from_groups_kernel, dim3((unsigned) ((n + 255) / 256)), dim3(256), 0, ctx->stream, d_seeds,
-                       d_group, d_representative, n);
+                       d_group, d_representative, (uint32_t) n_groups, n);
     return check_hip(hipGetLastError(), "seeds_from_groups_kernel launch");
 }
 

@@ -260,17 +260,22 @@ def test_device_block_cache_limit_and_trim(capi, ctx):
 
 
 def test_seeds_from_groups(capi, ctx):
-    """skm_seeds_from_groups: open entries (0xffffffff) take the representative of the point's group, the others stay."""
+    """skm_seeds_from_groups: open entries (0xffffffff) take the representative of the point's group, the others stay;
+    a group out of range counts as the last one."""
     g = np.random.default_rng(3)
     n, groups = 100_003, 37
     seeds = g.integers(0, 5000, n, dtype=np.uint32)
     seeds[g.random(n) < 0.7] = 0xFFFFFFFF
     group = g.integers(0, groups, n, dtype=np.uint32)
+    seeds[5] = seeds[77] = 0xFFFFFFFF
+    group[5], group[77] = groups, 0xFFFFFFF0
     rep = g.integers(0, 5000, groups, dtype=np.uint32)
     dS, dG, dR = ctx.array(seeds), ctx.array(group), ctx.array(rep)
-    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, n))
-    want = np.where(seeds == 0xFFFFFFFF, rep[group], seeds)
+    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, groups, n))
+    want = np.where(seeds == 0xFFFFFFFF, rep[np.minimum(group, groups - 1)], seeds)
     assert np.array_equal(dS.download(), want)
-    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, 0))
+    capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, groups, 0))
+    with pytest.raises(capi.SkmError):
+        capi.check(ctx.lib.skm_seeds_from_groups(ctx.handle, dS.ptr, dG.ptr, dR.ptr, 0, n))
     for a in (dS, dG, dR):
         a.free()
