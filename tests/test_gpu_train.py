@@ -406,8 +406,15 @@ def test_hierarchical_train_matches_oracle(capi, ctx, oracle, blobs, n, d, k):
     _, gbest, _ = oracle.brute_force(X, C)
     _, obest, _ = oracle.brute_force(X, OC)
     assert abs(gbest.sum() - obest.sum()) <= 1e-2 * obest.sum()
-    used = len(np.unique(km.assign(X, C)))
+    exact = km.assign(X, C)
+    used = len(np.unique(exact))
     assert used >= 0.95 * k  # test_hierarchical_superkmeans.cpp:554-587
+    # the pruned assignment of the training points from a hierarchical object: seeds are the assignments of its Train
+    # (sampling_fraction 1.0), its pruner tables hold the hierarchical threshold (test_assign.cpp:118-155 for the bar)
+    trained = km.assignments(n)
+    atp = km.assign_training_points(X, C)
+    assert np.mean(atp == exact) >= 0.98
+    assert np.array_equal(km.training_seeds(n), trained)
     km.close()
 
 
